@@ -1,0 +1,268 @@
+// Feed-forward parts of the layered models.
+//
+//   lgs_glu              out = act(a) * b over two column ranges of one projection (the dense gated feed-forward)
+//   lgs_moe_route        per token: the `top` largest router logits (fp32, lowest index first among equals) and the
+//                        softmax over just those
+//   lgs_moe_up / _down   the routed experts as streaming GEMVs over (token, choice) pairs: only the chosen experts'
+//                        rows are read; the down kernel sums a token's choices in their routing order and adds the
+//                        result to the residual stream (the decode form; a prompt runs grouped products instead)
+//   lgs_moe_sort / lgs_moe_combine   the prompt form: a stable counting sort of the (token, choice) pairs by
+//                        expert, whose ranges drive lgs_linear's grouped products, and the weighted sum back
+//   lgs_token_side       per-layer token input: x += unit_rms(proj(gelu_tanh(gate x) * e[token])) * w
+#include "seq_common.h"
+
+namespace lgs {
+
+__global__ void __launch_bounds__(256) glu_kernel(const float* __restrict__ a, const float* __restrict__ b, long ld,
+                                                  float* __restrict__ out, int n, int act) {
+  const size_t t = blockIdx.y;
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) out[t * n + i] = act_f(act, a[t * ld + i]) * b[t * ld + i];
+}
+
+// one wave per token; lane holds logits lane + 64 e (E <= 256)
+__global__ void __launch_bounds__(64) moe_route_kernel(const float* __restrict__ z, long ld, int E, int top,
+                                                       int* __restrict__ ids, float* __restrict__ wts) {
+  const int t = blockIdx.x, lane = threadIdx.x;
+  float v[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) v[e] = lane + 64 * e < E ? z[(size_t)t * ld + lane + 64 * e] : -INFINITY;
+  float first = 0.0f, den = 0.0f;
+  for (int k = 0; k < top; ++k) {
+    float best = -INFINITY;
+    int bi = 0x7fffffff;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int i = lane + 64 * e;
+      if (i < E && (v[e] > best || (v[e] == best && i < bi))) {
+        best = v[e];
+        bi = i;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ob = __shfl_xor(best, o);
+      const int oi = __shfl_xor(bi, o);
+      if (ob > best || (ob == best && oi < bi)) {
+        best = ob;
+        bi = oi;
+      }
+    }
+    if (k == 0) first = best;
+    const float w = expf(best - first);  // the first pick is the maximum
+    den += w;
+    if (lane == 0) {
+      ids[(size_t)t * top + k] = bi;
+      wts[(size_t)t * top + k] = w;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (lane + 64 * e == bi) v[e] = -INFINITY;
+  }
+  __syncthreads();
+  if (lane == 0)
+    for (int k = 0; k < top; ++k) wts[(size_t)t * top + k] /= den;
+}
+
+// grid (ceil(F / 8), pairs): pair = token * top + choice; act[pair][f] = act(up_e[f] . h_token)
+template <bool WF32>
+__global__ void __launch_bounds__(256) moe_up_kernel(const float* __restrict__ h, long ldh, const void* __restrict__ up,
+                                                     const int* __restrict__ ids, float* __restrict__ actbuf, int top,
+                                                     int F, int K, int act) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int pair = blockIdx.y, f0 = (blockIdx.x * 4 + wave) * 2;
+  if (f0 >= F) return;
+  const int e = ids[pair];
+  const float* hr = h + (size_t)(pair / top) * ldh;
+  const size_t w0 = ((size_t)e * F + f0) * K, w1 = ((size_t)e * F + min(f0 + 1, F - 1)) * K;
+  float a0 = 0.0f, a1 = 0.0f;
+  for (int k = lane; k < K; k += 64) {
+    const float x = aop<WF32>(hr[k]);
+    a0 = fmaf(x, wload<WF32>(up, w0 + k), a0);
+    a1 = fmaf(x, wload<WF32>(up, w1 + k), a1);
+  }
+  a0 = wave_sum(a0);
+  a1 = wave_sum(a1);
+  if (lane == 0) {
+    actbuf[(size_t)pair * F + f0] = act_f(act, a0);
+    if (f0 + 1 < F) actbuf[(size_t)pair * F + f0 + 1] = act_f(act, a1);
+  }
+}
+
+// grid (ceil(N / 8), T): x[t][n] += sum_k wts[t][k] * (down_e(t,k)[n] . act[t * top + k]), k ascending
+template <bool WF32>
+__global__ void __launch_bounds__(256) moe_down_kernel(const float* __restrict__ actbuf, const void* __restrict__ down,
+                                                       const int* __restrict__ ids, const float* __restrict__ wts,
+                                                       float* __restrict__ x, long ldx, int top, int N, int F) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int t = blockIdx.y, n0 = (blockIdx.x * 4 + wave) * 2;
+  if (n0 >= N) return;
+  float y0 = 0.0f, y1 = 0.0f;
+  for (int k = 0; k < top; ++k) {
+    const int e = ids[(size_t)t * top + k];
+    const float* ar = actbuf + ((size_t)t * top + k) * F;
+    const size_t w0 = ((size_t)e * N + n0) * F, w1 = ((size_t)e * N + min(n0 + 1, N - 1)) * F;
+    float a0 = 0.0f, a1 = 0.0f;
+    for (int f = lane; f < F; f += 64) {
+      const float a = aop<WF32>(ar[f]);
+      a0 = fmaf(a, wload<WF32>(down, w0 + f), a0);
+      a1 = fmaf(a, wload<WF32>(down, w1 + f), a1);
+    }
+    const float w = wts[(size_t)t * top + k];
+    y0 = fmaf(w, wave_sum(a0), y0);
+    y1 = fmaf(w, wave_sum(a1), y1);
+  }
+  if (lane == 0) {
+    x[(size_t)t * ldx + n0] += y0;
+    if (n0 + 1 < N) x[(size_t)t * ldx + n0 + 1] += y1;
+  }
+}
+
+// One workgroup: stable counting sort of the pairs by expert. z_start[E + 1] expert ranges in the sorted list,
+// tok_of[i] the token (row of h) of sorted entry i, where[pair] the sorted place of a pair.
+__global__ void __launch_bounds__(256) moe_sort_kernel(const int* __restrict__ ids, int pairs, int top, int E,
+                                                       int* __restrict__ z_start, int* __restrict__ tok_of,
+                                                       int* __restrict__ where) {
+  __shared__ int start[257];
+  const int tid = threadIdx.x;
+  // thread e counts expert e (E <= 256): a plain pass keeps the order stable and needs no atomics
+  int cnt = 0;
+  if (tid < E)
+    for (int i = 0; i < pairs; ++i) cnt += ids[i] == tid;
+  if (tid == 0) start[0] = 0;
+  __syncthreads();
+  // prefix over at most 256 counts by one thread per step would be slow; E is small, thread 0 scans
+  __shared__ int counts[256];
+  counts[tid] = tid < E ? cnt : 0;
+  __syncthreads();
+  if (tid == 0)
+    for (int e = 0; e < E; ++e) start[e + 1] = start[e] + counts[e];
+  __syncthreads();
+  if (tid < E) z_start[tid] = start[tid];
+  if (tid == 0) z_start[E] = start[E];
+  if (tid < E) {
+    int at = start[tid];
+    for (int i = 0; i < pairs; ++i)
+      if (ids[i] == tid) {
+        tok_of[at] = i / top;
+        where[i] = at;
+        ++at;
+      }
+  }
+}
+
+// grid (ceil(N / 256), T): x[t] += sum_k wts[t][k] * y[where[t * top + k]], k ascending
+__global__ void __launch_bounds__(256) moe_combine_kernel(const float* __restrict__ y, const int* __restrict__ where,
+                                                          const float* __restrict__ wts, float* __restrict__ x, long ldx,
+                                                          int top, int N) {
+  const int t = blockIdx.y, n = blockIdx.x * 256 + threadIdx.x;
+  if (n >= N) return;
+  float s = 0.0f;
+  for (int k = 0; k < top; ++k) s = fmaf(wts[(size_t)t * top + k], y[(size_t)where[(size_t)t * top + k] * N + n], s);
+  x[(size_t)t * ldx + n] += s;
+}
+
+// grid (T): LDS holds the row x (W floats), the gated slice (dim floats) and the projection y (W floats)
+template <bool WF32>
+__global__ void __launch_bounds__(256) token_side_kernel(float* __restrict__ x, const int* __restrict__ tok,
+                                                         const void* __restrict__ table, long ld_table, int col0,
+                                                         const void* __restrict__ gate_w, const void* __restrict__ proj_w,
+                                                         const float* __restrict__ norm_w, int W, int dim, int vocab,
+                                                         float eps) {
+  extern __shared__ float sh[];
+  __shared__ float red[4];
+  float* xs = sh;
+  float* ys = sh + W;
+  float* gs = sh + 2 * W;
+  const int t = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  float* xr = x + (size_t)t * W;
+  int id = tok[t];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  for (int i = tid; i < W; i += 256) xs[i] = aop<WF32>(xr[i]);
+  __syncthreads();
+  for (int j = wave; j < dim; j += 4) {
+    float a = 0.0f;
+    for (int k = lane; k < W; k += 64) a = fmaf(xs[k], wload<WF32>(gate_w, (size_t)j * W + k), a);
+    a = wave_sum(a);
+    if (lane == 0) gs[j] = aop<WF32>(gelu_tanh_f(a) * wload<WF32>(table, (size_t)id * ld_table + col0 + j));
+  }
+  __syncthreads();
+  float ss = 0.0f;
+  for (int n = tid; n < W; n += 256) {
+    float a = 0.0f;
+    for (int j = 0; j < dim; ++j) a = fmaf(gs[j], wload<WF32>(proj_w, (size_t)n * dim + j), a);
+    ys[n] = a;
+    ss = fmaf(a, a, ss);
+  }
+  ss = block_sum_256(ss, red);
+  const float rstd = 1.0f / sqrtf(ss / (float)W + eps);
+  for (int n = tid; n < W; n += 256) xr[n] += ys[n] * rstd * norm_w[n];
+}
+
+}  // namespace lgs
+
+extern "C" int lgs_glu(const float* a, const float* b, long ld, float* out, int T, int n, int act,
+                       hipStream_t stream) {
+  LGA_CHECK_ARG(a && b && out && T > 0 && T <= 65535 && n > 0, "lgs_glu: bad arguments");
+  lgs::glu_kernel<<<dim3((n + 255) / 256, T), 256, 0, stream>>>(a, b, ld, out, n, act);
+  LGA_LAUNCH_RETURN();
+}
+
+extern "C" int lgs_moe_route(const float* z, long ld, int T, int E, int top, int* ids, float* wts,
+                             hipStream_t stream) {
+  LGA_CHECK_ARG(z && ids && wts && T > 0, "lgs_moe_route: bad arguments");
+  LGA_CHECK_ARG(E > 0 && E <= 256 && top > 0 && top <= E, "lgs_moe_route: experts must be <= 256 and top <= experts");
+  lgs::moe_route_kernel<<<T, 64, 0, stream>>>(z, ld, E, top, ids, wts);
+  LGA_LAUNCH_RETURN();
+}
+
+extern "C" int lgs_moe_up(const float* h, long ldh, const void* up, int w_f32, const int* ids, float* actbuf, int T,
+                          int top, int F, int K, int act, hipStream_t stream) {
+  LGA_CHECK_ARG(h && up && ids && actbuf && T > 0 && top > 0 && F > 0 && K > 0 && (long)T * top <= 65535,
+                "lgs_moe_up: bad arguments");
+  const dim3 grid((F + 7) / 8, T * top);
+  if (w_f32) lgs::moe_up_kernel<true><<<grid, 256, 0, stream>>>(h, ldh, up, ids, actbuf, top, F, K, act);
+  else lgs::moe_up_kernel<false><<<grid, 256, 0, stream>>>(h, ldh, up, ids, actbuf, top, F, K, act);
+  LGA_LAUNCH_RETURN();
+}
+
+extern "C" int lgs_moe_down(const float* actbuf, const void* down, int w_f32, const int* ids, const float* wts,
+                            float* x, long ldx, int T, int top, int N, int F, hipStream_t stream) {
+  LGA_CHECK_ARG(actbuf && down && ids && wts && x && T > 0 && T <= 65535 && top > 0 && N > 0 && F > 0,
+                "lgs_moe_down: bad arguments");
+  const dim3 grid((N + 7) / 8, T);
+  if (w_f32) lgs::moe_down_kernel<true><<<grid, 256, 0, stream>>>(actbuf, down, ids, wts, x, ldx, top, N, F);
+  else lgs::moe_down_kernel<false><<<grid, 256, 0, stream>>>(actbuf, down, ids, wts, x, ldx, top, N, F);
+  LGA_LAUNCH_RETURN();
+}
+
+extern "C" int lgs_moe_sort(const int* ids, int pairs, int top, int E, int* z_start, int* tok_of, int* where,
+                            hipStream_t stream) {
+  LGA_CHECK_ARG(ids && z_start && tok_of && where && pairs > 0 && top > 0 && E > 0 && E <= 256,
+                "lgs_moe_sort: experts must be <= 256");
+  lgs::moe_sort_kernel<<<1, 256, 0, stream>>>(ids, pairs, top, E, z_start, tok_of, where);
+  LGA_LAUNCH_RETURN();
+}
+
+extern "C" int lgs_moe_combine(const float* y, const int* where, const float* wts, float* x, long ldx, int T, int top,
+                               int N, hipStream_t stream) {
+  LGA_CHECK_ARG(y && where && wts && x && T > 0 && T <= 65535 && top > 0 && N > 0, "lgs_moe_combine: bad arguments");
+  lgs::moe_combine_kernel<<<dim3((N + 255) / 256, T), 256, 0, stream>>>(y, where, wts, x, ldx, top, N);
+  LGA_LAUNCH_RETURN();
+}
+
+extern "C" int lgs_token_side(float* x, const int* tokens, const void* table, int w_f32, long ld_table, int col0,
+                              const void* gate_w, const void* proj_w, const float* norm_w, int T, int W, int dim,
+                              int vocab, float eps, hipStream_t stream) {
+  LGA_CHECK_ARG(x && tokens && table && gate_w && proj_w && norm_w && T > 0 && W > 0 && dim > 0 && vocab > 0,
+                "lgs_token_side: bad arguments");
+  const size_t lds = (size_t)(2 * W + dim) * sizeof(float);
+  LGA_CHECK_ARG(lds <= 64 * 1024, "lgs_token_side: width too large for one workgroup's LDS");
+  if (w_f32)
+    lgs::token_side_kernel<true><<<T, 256, lds, stream>>>(x, tokens, table, ld_table, col0, gate_w, proj_w, norm_w, W,
+                                                          dim, vocab, eps);
+  else
+    lgs::token_side_kernel<false><<<T, 256, lds, stream>>>(x, tokens, table, ld_table, col0, gate_w, proj_w, norm_w, W,
+                                                           dim, vocab, eps);
+  LGA_LAUNCH_RETURN();
+}

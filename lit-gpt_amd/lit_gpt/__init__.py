@@ -1,8 +1,8 @@
 """MI355X-native decode path behind the lit_gpt API (reference lit_gpt/__init__.py:27)."""
 
-from lit_gpt.config import Config
+from lit_gpt.config import Config, LayeredConfig, load_config, model_class
 
-__all__ = ["GPT", "Config", "Tokenizer"]
+__all__ = ["GPT", "Config", "LayeredConfig", "LayeredGPT", "Tokenizer", "load_config", "model_class"]
 
 
 def __getattr__(name):
@@ -10,6 +10,10 @@ def __getattr__(name):
         from lit_gpt.model import GPT
 
         return GPT
+    if name == "LayeredGPT":
+        from lit_gpt.layered import LayeredGPT
+
+        return LayeredGPT
     if name == "Tokenizer":
         from lit_gpt.tokenizer import Tokenizer
 

@@ -159,3 +159,149 @@ for _kind in ("", "Instruct-"):
               rope_base=1000000, n_expert=8, n_expert_per_token=2)
 
 name_to_config: Dict[str, Dict[str, Any]] = {c["name"]: c for c in configs}
+
+
+# --------------------------------------------------------------------------------------------
+# Layered models: a ``config.json`` that lists its layers one by one (each with its own sequence mixer and
+# feed-forward) instead of repeating one block. ``architecture`` names the design; the registry below maps it to
+# the model class, and ``load_config`` picks the configuration class for a checkpoint folder.
+# --------------------------------------------------------------------------------------------
+@dataclass
+class RotarySpec:
+    dims: int = 0
+    base: float = 10000.0
+
+    def inv_freq(self) -> List[float]:
+        """f_i = base^(-2i / dims), i < dims / 2, in double precision (rounded once to fp32 by the caller)."""
+        return [float(self.base) ** (-2.0 * i / self.dims) for i in range(self.dims // 2)]
+
+
+@dataclass
+class MixerSpec:
+    kind: str  # "retention" | "latent_attention"
+    heads: int
+    dim: int  # per-head query / key size (latent attention: the unrotated part)
+    vdim: int
+    rot: RotarySpec
+    decay: Optional[List[float]] = None  # retention: one fixed decay per head
+    kv_rank: int = 0  # latent attention: size of the cached latent
+    rot_dim: int = 0  # latent attention: rotated query / key part (one key part shared by the heads)
+    scale: float = 1.0  # latent attention: score scale
+
+
+@dataclass
+class FeedForwardSpec:
+    kind: str  # "dense" | "moe"
+    ff: int
+    experts: int = 0
+    top: int = 0
+
+
+@dataclass
+class LayerSpec:
+    mixer: MixerSpec
+    mlp: Optional[FeedForwardSpec]
+
+
+MIXER_KINDS = ("retention", "latent_attention")
+
+
+@dataclass
+class LayeredConfig:
+    architecture: str
+    vocab: int
+    width: int
+    norm_eps: float
+    embedding_scale: float
+    layers: List[LayerSpec]
+    loop_start: int = 0
+    loop_stop: int = 0
+    loop_times: int = 1
+    side_dim: int = 0  # per-layer token input: width of each layer's slice of the second embedding table (0: none)
+    name: str = ""
+
+    def __post_init__(self) -> None:
+        self.name = self.name or self.architecture
+        n = len(self.layers)
+        if not (0 <= self.loop_start <= self.loop_stop <= n) or self.loop_times < 1:
+            raise ValueError(f"loop [{self.loop_start}, {self.loop_stop}) x {self.loop_times} does not fit {n} layers")
+        for i, spec in enumerate(self.layers):
+            m = spec.mixer
+            if m.kind not in MIXER_KINDS:
+                raise ValueError(f"layer {i}: unknown mixer {m.kind!r}")
+            if m.kind == "retention" and (m.decay is None or len(m.decay) != m.heads):
+                raise ValueError(f"layer {i}: retention needs one decay per head")
+            if m.rot.dims % 2 or m.rot.dims > (m.rot_dim if m.kind == "latent_attention" else m.dim):
+                raise ValueError(f"layer {i}: rotary dims {m.rot.dims} do not fit the head")
+            if spec.mlp is not None and spec.mlp.kind == "moe" and not 0 < spec.mlp.top <= spec.mlp.experts:
+                raise ValueError(f"layer {i}: top {spec.mlp.top} of {spec.mlp.experts} experts")
+
+    @property
+    def layer_runs(self) -> List[int]:
+        """Layer index of every layer run in order: layers [loop_start, loop_stop) run loop_times times in a row
+        with the same weights (each run with a cache or state of its own), the others once."""
+        a, b = self.loop_start, self.loop_stop
+        return list(range(a)) + list(range(a, b)) * self.loop_times + list(range(b, len(self.layers)))
+
+    @classmethod
+    def from_dict(cls, d: Dict[str, Any]) -> "LayeredConfig":
+        layers = []
+        for entry in d["layers"]:
+            m = entry["mixer"]
+            rot = m.get("rot") or {}
+            mixer = MixerSpec(kind=entry["type"], heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                              rot=RotarySpec(int(rot.get("dims", 0)), float(rot.get("base", 10000.0))),
+                              decay=[float(x) for x in m["decay"]] if "decay" in m else None,
+                              kv_rank=int(m.get("kv_rank", 0)), rot_dim=int(m.get("rot_dim", 0)),
+                              scale=float(m.get("scale", 1.0)))
+            f = entry.get("mlp")
+            if f is None:
+                mlp = None
+            elif f["kind"] == "dense":
+                mlp = FeedForwardSpec("dense", int(f["ff"]))
+            elif f["kind"] == "moe":
+                mlp = FeedForwardSpec("moe", int(f["expert"]["ff"]), int(f["router"]["experts"]), int(f["router"]["top"]))
+            else:
+                raise ValueError(f"unknown feed-forward kind {f['kind']!r}")
+            layers.append(LayerSpec(mixer, mlp))
+        loop = d.get("loop") or {}
+        side = d.get("token_side") or {}
+        return cls(architecture=d["architecture"], vocab=int(d["vocab"]), width=int(d["width"]),
+                   norm_eps=float(d["norm"]["eps"]), embedding_scale=float((d.get("embedding") or {}).get("scale", 1.0)),
+                   layers=layers, loop_start=int(loop.get("start", 0)), loop_stop=int(loop.get("stop", 0)),
+                   loop_times=int(loop.get("times", 1)), side_dim=int(side.get("dim", 0)))
+
+    @classmethod
+    def from_json(cls, path: Union[str, Path]) -> "LayeredConfig":
+        with open(path, encoding="utf-8") as fp:
+            return cls.from_dict(json.load(fp))
+
+
+# architecture name (config.json) -> "module:class" of the model that serves it
+ARCHITECTURES: Dict[str, str] = {"Bavesun": "lit_gpt.layered:LayeredGPT"}
+
+
+def load_config(checkpoint_dir: Union[str, Path]) -> Union[Config, LayeredConfig]:
+    """The configuration of a checkpoint folder: ``config.json`` with a registered ``architecture`` gives a
+    LayeredConfig, anything else goes through ``Config.from_checkpoint`` (lit_config.json or a registered name)."""
+    path = Path(checkpoint_dir)
+    cj = path / "config.json"
+    if cj.is_file():
+        with open(cj, encoding="utf-8") as fp:
+            d = json.load(fp)
+        if d.get("architecture") in ARCHITECTURES:
+            return LayeredConfig.from_dict(d)
+        if "architecture" in d and not (path / "lit_config.json").is_file():
+            raise ValueError(f"architecture {d['architecture']!r} is not registered (known: {sorted(ARCHITECTURES)})")
+    return Config.from_checkpoint(path)
+
+
+def model_class(config: Union[Config, LayeredConfig]) -> Type:
+    if isinstance(config, LayeredConfig):
+        import importlib
+
+        mod, _, cls = ARCHITECTURES[config.architecture].partition(":")
+        return getattr(importlib.import_module(mod), cls)
+    import lit_gpt.model
+
+    return lit_gpt.model.GPT

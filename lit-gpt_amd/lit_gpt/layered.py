@@ -1,0 +1,245 @@
+"""LayeredGPT: a decoder whose ``config.json`` lists its layers one by one, each with its own sequence mixer
+(``lit_gpt.mixers``) and feed-forward, optionally looping a range of layers with shared weights.
+
+It keeps the serving surface of ``lit_gpt.GPT`` — ``forward(idx, input_pos)``, ``max_seq_length``,
+``set_kv_cache`` / ``clear_kv_cache`` — so ``generate.base.generate`` drives it unchanged, and adds the packed-batch
+step (``forward_step`` / ``logits``) that ``generate.batch.BatchEngine`` schedules. The residual stream, norms,
+attention scores, recurrent states and routers are fp32 in both precisions; ``dtype`` (bf16 or fp32) is the dtype
+of the weight matrices and of the cached latent, and picks bf16-operand / fp32-sum products or plain fp32 ones.
+
+A layer is parallel: h = norm(x); x <- x + mixer(h) + ff(h); then the optional per-layer token input. The norm's
+weight is stored around zero (offset 1). Every matrix that reads h is one row block of a single fused input
+projection. Logits come from the embedding table itself (tied, unscaled) after the final norm.
+"""
+
+from __future__ import annotations
+
+from pathlib import Path
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+import torch.nn as nn
+
+from lit_gpt import seq_ops
+from lit_gpt.config import LayeredConfig, LayerSpec
+from lit_gpt.mixers import MIXERS, GatedFeedForward, SparseFeedForward, StepBatch, TokenSide
+from lit_gpt.rmsnorm import StreamRMSNorm
+
+
+def _sub(w: Dict[str, torch.Tensor], prefix: str) -> Dict[str, torch.Tensor]:
+    return {k[len(prefix):]: v for k, v in w.items() if k.startswith(prefix)}
+
+
+class LayeredBlock(nn.Module):
+    def __init__(self, index: int, spec: LayerSpec, config: LayeredConfig, w: Dict[str, torch.Tensor],
+                 side_table: Optional[torch.Tensor], device, dtype) -> None:
+        super().__init__()
+        W, eps = config.width, config.norm_eps
+        self.norm1 = StreamRMSNorm(W, eps=eps, offset=1.0)
+        self.norm1.weight = w["norm1"].to(device=device, dtype=torch.float32).contiguous()
+        self.mixer = MIXERS[spec.mixer.kind](spec.mixer, W, eps, _sub(w, "mix."), device, dtype)
+        self.mlp = None
+        if spec.mlp is not None:
+            cls = GatedFeedForward if spec.mlp.kind == "dense" else SparseFeedForward
+            self.mlp = cls(spec.mlp, W, _sub(w, "mlp."), device, dtype)
+        self.side = None
+        if side_table is not None and "side.gate" in w:
+            self.side = TokenSide(index, config.side_dim, side_table, _sub(w, "side."), eps, device, dtype)
+        # one input projection for everything that reads the norm's output
+        parts, offsets, at = [], [{}, {}], 0
+        for k, mod in enumerate((self.mixer, self.mlp)):
+            if mod is None:
+                continue
+            for name, t in mod.in_parts():
+                offsets[k][name] = at
+                parts.append(t)
+                at += t.shape[0]
+                pad = -at % 8  # every part starts on a 32-byte boundary of the fp32 row
+                if pad:
+                    parts.append(torch.zeros(pad, W, dtype=t.dtype))
+                    at += pad
+        self.mixer.bind(offsets[0])
+        if self.mlp is not None:
+            self.mlp.bind(offsets[1])
+        self.register_buffer("w_in", torch.cat(parts).to(device=device, dtype=dtype).contiguous())
+
+    def forward(self, x: torch.Tensor, step: StepBatch, cache: nn.Module) -> None:
+        """x (T, width) fp32, updated in place."""
+        h = self.norm1(x)
+        n_in, W = self.w_in.shape
+        proj = torch.empty(step.T, n_in, dtype=torch.float32, device=x.device)
+        seq_ops.linear(h, self.w_in, M=step.T, N=n_in, K=W, y=proj, lda=W, ldy=n_in)
+        self.mixer(proj, step, cache, x)
+        if self.mlp is not None:
+            self.mlp(proj, h, x)
+        if self.side is not None:
+            self.side(x, step.tokens)
+
+
+class LayeredGPT(nn.Module):
+    decode_graph = False  # generate.base.generate steps this model eagerly (its graph executor is GPT's)
+
+    def __init__(self, config: LayeredConfig, weights: Dict[str, torch.Tensor], *, device: torch.device,
+                 dtype: torch.dtype = torch.bfloat16) -> None:
+        super().__init__()
+        if dtype not in (torch.bfloat16, torch.float32):
+            raise NotImplementedError(f"dtype {dtype}: the MI355X path computes with bf16 or fp32 weights")
+        if torch.device(device).type != "cuda":
+            raise RuntimeError("LayeredGPT: this build computes on the MI355X only (no CPU path)")
+        self.config, self.dtype, self.device = config, dtype, torch.device(device)
+        V, W = config.vocab, config.width
+        if tuple(weights["embed"].shape) != (V, W):
+            raise ValueError(f"embed: shape {tuple(weights['embed'].shape)}, expected {(V, W)}")
+        self.register_buffer("embed", weights["embed"].to(device=device, dtype=dtype).contiguous())
+        self.register_buffer("side_embed", None)
+        if config.side_dim:
+            t = weights["side.embed"]
+            if t.shape[0] != V or t.shape[1] < config.side_dim * len(config.layers):
+                raise ValueError(f"side.embed: shape {tuple(t.shape)} does not hold {len(config.layers)} slices")
+            self.side_embed = t.to(device=device, dtype=dtype).contiguous()
+        self.blocks = nn.ModuleList(
+            LayeredBlock(i, spec, config, _sub(weights, f"l{i}."), self.side_embed, device, dtype)
+            for i, spec in enumerate(config.layers))
+        self.final_norm = StreamRMSNorm(W, eps=config.norm_eps, offset=1.0)
+        self.final_norm.weight = weights["final.norm"].to(device=device, dtype=torch.float32).contiguous()
+        self.runs: List[int] = config.layer_runs
+        self.caches: Optional[nn.ModuleList] = None  # one cache / state per layer run
+        self._max_seq_length = 0
+        self.eval()
+
+    # ------------------------------------------------------------------------------------------ construction
+    @classmethod
+    def from_checkpoint(cls, checkpoint_dir, *, device, dtype=torch.bfloat16) -> "LayeredGPT":
+        """``config.json`` + ``model.safetensors`` (bf16 matrices [out, in], names l<i>.mix.* / .mlp.* / .side.*)."""
+        from lit_gpt.utils import read_safetensors
+
+        path = Path(checkpoint_dir)
+        config = LayeredConfig.from_json(path / "config.json")
+        return cls(config, read_safetensors(path / "model.safetensors"), device=device, dtype=dtype)
+
+    @staticmethod
+    def tensor_shapes(config: LayeredConfig) -> Dict[str, Tuple[int, ...]]:
+        """Name -> shape of every checkpoint tensor of a configuration."""
+        W, out = config.width, {"embed": (config.vocab, config.width), "final.norm": (config.width,)}
+        if config.side_dim:
+            out["side.embed"] = (config.vocab, config.side_dim * len(config.layers))
+        for i, spec in enumerate(config.layers):
+            m, p = spec.mixer, f"l{i}."
+            out[p + "norm1"] = (W,)
+            if m.kind == "retention":
+                out.update({p + "mix.q": (m.heads * m.dim, W), p + "mix.k": (m.heads * m.dim, W),
+                            p + "mix.v": (m.heads * m.vdim, W), p + "mix.g": (m.heads * m.vdim, W),
+                            p + "mix.o": (W, m.heads * m.vdim)})
+            else:
+                out.update({p + "mix.q": (m.heads * (m.dim + m.rot_dim), W), p + "mix.dkv": (m.kv_rank + m.rot_dim, W),
+                            p + "mix.dkv.norm": (m.kv_rank,), p + "mix.uk": (m.heads * m.dim, m.kv_rank),
+                            p + "mix.uv": (m.heads * m.vdim, m.kv_rank), p + "mix.sink": (m.heads,),
+                            p + "mix.g": (m.heads * m.vdim, W), p + "mix.o": (W, m.heads * m.vdim)})
+            f = spec.mlp
+            if f is not None and f.kind == "dense":
+                out.update({p + "mlp.gate": (f.ff, W), p + "mlp.up": (f.ff, W), p + "mlp.down": (W, f.ff)})
+            elif f is not None:
+                out[p + "mlp.router"] = (f.experts, W)
+                for e in range(f.experts):
+                    out.update({p + f"mlp.e{e}.up": (f.ff, W), p + f"mlp.e{e}.down": (W, f.ff)})
+            if config.side_dim:
+                out.update({p + "side.gate": (config.side_dim, W), p + "side.proj": (W, config.side_dim),
+                            p + "side.norm": (W,)})
+        return out
+
+    @classmethod
+    def random_weights(cls, config: LayeredConfig, seed: int = 0) -> Dict[str, torch.Tensor]:
+        """Random bf16 checkpoint tensors (matrices ~ N(0, 1/fan_in), norm weights small, sinks ~ N(0, 1))."""
+        g = torch.Generator().manual_seed(seed)
+        out = {}
+        for name, shape in cls.tensor_shapes(config).items():
+            if name.endswith("norm1") or name == "final.norm":
+                t = 0.1 * torch.randn(shape, generator=g)
+            elif name.endswith(".norm"):
+                t = 1.0 + 0.1 * torch.randn(shape, generator=g)
+            elif name.endswith("sink"):
+                t = torch.randn(shape, generator=g)
+            elif name.endswith("embed"):
+                t = torch.randn(shape, generator=g) * (1.0 if name == "side.embed" else shape[1] ** -0.5)
+            else:
+                t = torch.randn(shape, generator=g) * shape[1] ** -0.5
+            out[name] = t.to(torch.bfloat16)
+        return out
+
+    # ------------------------------------------------------------------------------------------ cache
+    @property
+    def max_seq_length(self) -> int:
+        return self._max_seq_length
+
+    @max_seq_length.setter
+    def max_seq_length(self, value: int) -> None:
+        if self.caches is not None and value != self._max_seq_length:
+            self.caches = None  # rebuilt by the next set_kv_cache
+        self._max_seq_length = int(value)
+
+    def set_kv_cache(self, batch_size: int, max_seq_length: Optional[int] = None,
+                     device: Optional[torch.device] = None, dtype: Optional[torch.dtype] = None) -> None:
+        """Caches and states for ``batch_size`` slots of ``max_seq_length`` positions, one per layer run."""
+        if max_seq_length is not None:
+            self.max_seq_length = max_seq_length
+        if self._max_seq_length <= 0:
+            raise ValueError("set max_seq_length (or pass it) before set_kv_cache")
+        self.caches = nn.ModuleList(
+            self.blocks[i].mixer.build_cache(batch_size, self._max_seq_length, device or self.device,
+                                             dtype or self.dtype) for i in self.runs)
+
+    def clear_kv_cache(self) -> None:
+        self.caches = None
+
+    @property
+    def slots(self) -> int:
+        return 0 if self.caches is None else self.caches[0].slots
+
+    def grow_slots(self, slots: int) -> None:
+        for c in self.caches:
+            c.grow(slots)
+
+    # ------------------------------------------------------------------------------------------ forward
+    @torch.inference_mode()
+    def forward_step(self, step: StepBatch) -> torch.Tensor:
+        """Run the step's tokens through every layer run from the caches and states earlier steps left; returns the
+        final residual stream (T, width) fp32 (before the final norm)."""
+        if self.caches is None:
+            raise TypeError("You need to call `set_kv_cache()`")
+        x = seq_ops.embed(step.tokens, self.embed, self.config.embedding_scale)
+        for run, layer in enumerate(self.runs):
+            self.blocks[layer](x, step, self.caches[run])
+        return x
+
+    @torch.inference_mode()
+    def logits(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Final norm and the tied output product for the given rows of the stream (int32 indices; all if None)."""
+        if rows is not None:
+            x = seq_ops.gather_rows(x, rows)
+        h = self.final_norm(x)
+        V, W = self.embed.shape
+        out = torch.empty(h.shape[0], V, dtype=torch.float32, device=h.device)
+        return seq_ops.linear(h, self.embed, M=h.shape[0], N=V, K=W, y=out, lda=W, ldy=V)
+
+    def forward(self, idx: torch.Tensor, input_pos: Optional[torch.Tensor] = None, *,
+                last_token_only: bool = False) -> torch.Tensor:
+        """``GPT.forward``'s contract for one sequence in slot 0: (1, T) ids at positions ``input_pos`` (consecutive;
+        default 0..T-1, which starts the sequence anew) -> (1, T, vocab) fp32 logits, or (1, 1, vocab)."""
+        B, T = idx.shape
+        if B != 1:
+            raise NotImplementedError("forward() serves one sequence; batches go through generate.batch.BatchEngine")
+        dev = idx.device
+        if self.caches is None:
+            if input_pos is not None:
+                raise TypeError("You need to call `set_kv_cache()`")
+            self.set_kv_cache(1, max(T, self._max_seq_length))
+        if T > self._max_seq_length:
+            raise ValueError(f"Cannot forward sequence of length {T}, max seq length is only {self._max_seq_length}.")
+        pos = (torch.arange(T, device=dev) if input_pos is None else input_pos.to(dev)).to(torch.int32).contiguous()
+        zero = torch.zeros(1, dtype=torch.int32, device=dev)
+        step = StepBatch(idx.reshape(-1).to(torch.int32).contiguous(), zero.expand(T).contiguous(), pos,
+                         torch.tensor([0, T], dtype=torch.int32, device=dev), zero, pos[:1], T=T, B=1)
+        x = self.forward_step(step)
+        if last_token_only:
+            x = x[-1:].contiguous()
+        return self.logits(x).unsqueeze(0)

@@ -1,0 +1,246 @@
+"""Sequence mixers, feed-forwards and the per-layer token input of the layered models, on ``liblitgpt_seq.so``.
+
+Every module here reads one shared input projection: a layer's norm output ``h`` goes through ONE product with the
+row-wise concatenation of all the matrices that read it (the mixer's q / k / v / gate or q / latent / gate, the dense
+gate and up matrices, the router), and each module finds its columns in the result by offset. ``in_parts`` lists a
+module's rows of that matrix, ``bind`` tells it where they landed. Outputs are accumulated into the fp32 residual
+stream ``x`` by the epilogue of the out-projection (or the expert combine), so a layer needs no add kernel.
+
+A step is a packed batch (``StepBatch``): the tokens of all sequences row after row, with per-token cache slot and
+position and per-sequence row range, slot and first position, all int32 on the device. Sizes, decays, scales, rotary
+dims / bases and layouts are constructor parameters; nothing is fixed to one model.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+import torch.nn as nn
+
+from lit_gpt import seq_ops
+from lit_gpt.config import FeedForwardSpec, MixerSpec
+from lit_gpt.model import LatentKVCache, RetentionState
+
+
+@dataclass
+class StepBatch:
+    tokens: torch.Tensor  # (T,) int32
+    slot: torch.Tensor  # (T,) cache slot of each token's sequence
+    pos: torch.Tensor  # (T,) position of each token in its sequence
+    seq_start: torch.Tensor  # (B + 1,) first row of each sequence, then T
+    seq_slot: torch.Tensor  # (B,)
+    seq_pos0: torch.Tensor  # (B,) position of each sequence's first row
+    T: int
+    B: int
+
+    @classmethod
+    def build(cls, entries: Sequence[Tuple[int, int, Sequence[int]]], device: torch.device) -> "StepBatch":
+        """entries: (slot, first position, token ids) per sequence; one host -> device copy for the whole table."""
+        tokens, slot, pos, start, sslot, spos = [], [], [], [0], [], []
+        for s, p0, toks in entries:
+            n = len(toks)
+            if n == 0:
+                raise ValueError("a sequence brings no tokens to this step")
+            tokens += list(toks)
+            slot += [s] * n
+            pos += range(p0, p0 + n)
+            start.append(start[-1] + n)
+            sslot.append(s)
+            spos.append(p0)
+        T, B = len(tokens), len(entries)
+        flat = torch.tensor(tokens + slot + pos + start + sslot + spos, dtype=torch.int32).to(device)
+        cut = [T, T, T, B + 1, B, B]
+        parts = torch.split(flat, cut)
+        return cls(*parts, T=T, B=B)
+
+
+def _f32(t: torch.Tensor, device) -> torch.Tensor:
+    return t.to(device=device, dtype=torch.float32).contiguous()
+
+
+class InputReader(nn.Module):
+    """A module that reads columns of the layer's shared input projection."""
+
+    def in_parts(self) -> List[Tuple[str, torch.Tensor]]:
+        raise NotImplementedError
+
+    def bind(self, offsets: Dict[str, int]) -> None:
+        self.off = dict(offsets)
+
+
+class Retention(InputReader):
+    """Decayed linear attention without softmax or denominator: per head S_t = decay S_{t-1} + k_t v_t^T,
+    o_t = S_t^T q_t, rotary positions (pairs i, i + dims/2) on q and k, k scaled by ``k_scale``; each head's output is
+    divided by its root mean square, gated with silu(W_g h) and projected."""
+
+    def __init__(self, spec: MixerSpec, width: int, eps: float, w: Dict[str, torch.Tensor], device, dtype) -> None:
+        super().__init__()
+        self.H, self.d, self.dv, self.eps = spec.heads, spec.dim, spec.vdim, eps
+        self.rot_dims = spec.rot.dims
+        self.k_scale = float(spec.dim) ** -0.5
+        H, d, dv = self.H, self.d, self.dv
+        for name, rows in (("q", H * d), ("k", H * d), ("v", H * dv), ("g", H * dv)):
+            if tuple(w[name].shape) != (rows, width):
+                raise ValueError(f"retention.{name}: shape {tuple(w[name].shape)}, expected {(rows, width)}")
+        self._in = [(n, w[n]) for n in ("q", "k", "v", "g")]
+        self.register_buffer("w_o", w["o"].to(device=device, dtype=dtype).contiguous())
+        self.register_buffer("decay", torch.tensor(spec.decay, dtype=torch.float64).to(device=device, dtype=torch.float32))
+        self.register_buffer("inv_freq", torch.tensor(spec.rot.inv_freq() or [1.0], dtype=torch.float64)
+                             .to(device=device, dtype=torch.float32))
+
+    def in_parts(self):
+        return self._in
+
+    def build_cache(self, slots: int, max_seq_length: int, device, dtype) -> RetentionState:
+        return RetentionState(slots, self.H, self.d, self.dv, device=device)
+
+    def forward(self, proj: torch.Tensor, step: StepBatch, cache: RetentionState, x: torch.Tensor) -> None:
+        H, dv = self.H, self.dv
+        o = seq_ops.retention(proj, self.off["q"], self.off["k"], self.off["v"], cache.s, self.decay, self.inv_freq,
+                              step.seq_start, step.seq_slot, step.seq_pos0, H=H, d=self.d, dv=dv,
+                              rot_dims=self.rot_dims, k_scale=self.k_scale)
+        seq_ops.head_gate(o, proj, self.off["g"], H=H, dv=dv, unit_norm=True, eps=self.eps, act=seq_ops.ACT_SILU)
+        W = x.shape[1]
+        seq_ops.linear(o, self.w_o, M=step.T, N=W, K=H * dv, y=x, lda=H * dv, ldy=W, accumulate=True)
+
+
+class LatentAttention(InputReader):
+    """Causal softmax attention whose keys and values are expanded from a cached low-rank latent c (RMS-normed) and
+    one rotated key part shared by all heads (interleaved rotary pairs 2i, 2i + 1). The score of head h is
+    (q_h . W_uk,h c + q_rot,h . k_rot) * scale; the denominator also holds exp(sink_h). The kernels never expand
+    keys or values: the query is mapped through W_uk,h first (one product per head), attention runs over the cached
+    rows [c | k_rot] for all heads alike, and W_uv,h maps the weighted latent back. Output gate sigmoid(W_g h)."""
+
+    def __init__(self, spec: MixerSpec, width: int, eps: float, w: Dict[str, torch.Tensor], device, dtype) -> None:
+        super().__init__()
+        self.H, self.d, self.dr, self.dv, self.r = spec.heads, spec.dim, spec.rot_dim, spec.vdim, spec.kv_rank
+        self.eps, self.scale, self.rot_dims, self.dtype = eps, spec.scale, spec.rot.dims, dtype
+        H, d, dr, dv, r = self.H, self.d, self.dr, self.dv, self.r
+        for name, shape in (("q", (H * (d + dr), width)), ("dkv", (r + dr, width)), ("g", (H * dv, width)),
+                            ("uk", (H * d, r)), ("uv", (H * dv, r)), ("o", (width, H * dv))):
+            if tuple(w[name].shape) != shape:
+                raise ValueError(f"latent_attention.{name}: shape {tuple(w[name].shape)}, expected {shape}")
+        self._in = [(n, w[n]) for n in ("q", "dkv", "g")]
+        # per head (r, d): the key up-projection transposed, so that q_h (d values) maps to r latent coordinates
+        self.register_buffer("w_ukT", w["uk"].to(device=device, dtype=dtype).view(H, d, r).transpose(1, 2).contiguous())
+        self.register_buffer("w_uv", w["uv"].to(device=device, dtype=dtype).contiguous())
+        self.register_buffer("w_o", w["o"].to(device=device, dtype=dtype).contiguous())
+        self.register_buffer("norm_w", _f32(w["dkv.norm"], device))
+        self.register_buffer("sink", _f32(w["sink"], device) if "sink" in w else None)
+        self.register_buffer("inv_freq", torch.tensor(spec.rot.inv_freq() or [1.0], dtype=torch.float64)
+                             .to(device=device, dtype=torch.float32))
+
+    def in_parts(self):
+        return self._in
+
+    def build_cache(self, slots: int, max_seq_length: int, device, dtype) -> LatentKVCache:
+        return LatentKVCache(slots, max_seq_length, self.r, self.dr, device=device, dtype=dtype)
+
+    def forward(self, proj: torch.Tensor, step: StepBatch, cache: LatentKVCache, x: torch.Tensor) -> None:
+        H, d, dr, dv, r = self.H, self.d, self.dr, self.dv, self.r
+        T, ld = proj.shape
+        q_off = self.off["q"]
+        seq_ops.latent_prepare(proj, q_off, self.off["dkv"], cache.c, cache.kr, self.norm_w, self.inv_freq, step.slot,
+                               step.pos, H=H, d=d, dr=dr, r=r, rot_dims=self.rot_dims, eps=self.eps)
+        qc = torch.empty(T, H * r, dtype=torch.float32, device=proj.device)
+        seq_ops.linear(proj, self.w_ukT, M=T, N=r, K=d, y=qc, a_off=q_off, lda=ld, ldy=H * r, batch=H,
+                       stride_a=d + dr, stride_w=r * d, stride_y=r)
+        lat = seq_ops.latent_attention(qc, proj, q_off, cache.c, cache.kr, self.sink, step.slot, step.pos, H=H, d=d,
+                                       dr=dr, r=r, scale=self.scale)
+        att = torch.empty(T, H * dv, dtype=torch.float32, device=proj.device)
+        seq_ops.linear(lat, self.w_uv, M=T, N=dv, K=r, y=att, lda=H * r, ldy=H * dv, batch=H, stride_a=r,
+                       stride_w=dv * r, stride_y=dv)
+        seq_ops.head_gate(att, proj, self.off["g"], H=H, dv=dv, unit_norm=False, eps=self.eps,
+                          act=seq_ops.ACT_SIGMOID)
+        W = x.shape[1]
+        seq_ops.linear(att, self.w_o, M=T, N=W, K=H * dv, y=x, lda=H * dv, ldy=W, accumulate=True)
+
+
+class GatedFeedForward(InputReader):
+    """W_down (act(W_gate h) * (W_up h)); ``act`` one of seq_ops.ACT_*."""
+
+    def __init__(self, spec: FeedForwardSpec, width: int, w: Dict[str, torch.Tensor], device, dtype,
+                 act: int = seq_ops.ACT_GELU_TANH) -> None:
+        super().__init__()
+        self.ff, self.act = spec.ff, act
+        for name, shape in (("gate", (spec.ff, width)), ("up", (spec.ff, width)), ("down", (width, spec.ff))):
+            if tuple(w[name].shape) != shape:
+                raise ValueError(f"mlp.{name}: shape {tuple(w[name].shape)}, expected {shape}")
+        self._in = [("gate", w["gate"]), ("up", w["up"])]
+        self.register_buffer("w_down", w["down"].to(device=device, dtype=dtype).contiguous())
+
+    def in_parts(self):
+        return self._in
+
+    def forward(self, proj: torch.Tensor, h: torch.Tensor, x: torch.Tensor) -> None:
+        a = seq_ops.glu(proj, self.off["gate"], self.off["up"], self.ff, self.act)
+        W = x.shape[1]
+        seq_ops.linear(a, self.w_down, M=a.shape[0], N=W, K=self.ff, y=x, lda=self.ff, ldy=W, accumulate=True)
+
+
+class SparseFeedForward(InputReader):
+    """Mixture of experts: fp32 router logits, the ``top`` largest chosen, weights = softmax over the chosen logits
+    only, expert = W_down act(W_up h) without biases (``act`` defaults to the square of relu).
+
+    Few (token, choice) pairs (decode) stream only the chosen experts' rows through two GEMV launches. A prompt
+    sorts its pairs by expert on the device and runs two grouped products over the expert ranges, then sums each
+    token's choices in routing order."""
+
+    STREAM_PAIRS = 48  # up to this many (token, choice) pairs the streaming form runs
+
+    def __init__(self, spec: FeedForwardSpec, width: int, w: Dict[str, torch.Tensor], device, dtype,
+                 act: int = seq_ops.ACT_RELU2) -> None:
+        super().__init__()
+        self.E, self.top, self.ff, self.act = spec.experts, spec.top, spec.ff, act
+        if tuple(w["router"].shape) != (spec.experts, width):
+            raise ValueError(f"mlp.router: shape {tuple(w['router'].shape)}, expected {(spec.experts, width)}")
+        self._in = [("router", w["router"])]
+        up = torch.stack([w[f"e{e}.up"] for e in range(self.E)])
+        down = torch.stack([w[f"e{e}.down"] for e in range(self.E)])
+        if tuple(up.shape) != (self.E, spec.ff, width) or tuple(down.shape) != (self.E, width, spec.ff):
+            raise ValueError("mlp experts: unexpected shapes")
+        self.register_buffer("w_up", up.to(device=device, dtype=dtype).contiguous())
+        self.register_buffer("w_down", down.to(device=device, dtype=dtype).contiguous())
+
+    def in_parts(self):
+        return self._in
+
+    def forward(self, proj: torch.Tensor, h: torch.Tensor, x: torch.Tensor) -> None:
+        T, W = h.shape
+        E, top, F = self.E, self.top, self.ff
+        ids, wts = seq_ops.moe_route(proj, self.off["router"], E, top)
+        if T * top <= self.STREAM_PAIRS:
+            a = seq_ops.moe_up(h, self.w_up, ids, self.act)
+            seq_ops.moe_down(a, self.w_down, ids, wts, x)
+            return
+        pairs = T * top
+        z_start, tok_of, where = seq_ops.moe_sort(ids, E)
+        a = torch.empty(pairs, F, dtype=torch.float32, device=h.device)
+        seq_ops.linear(h, self.w_up, M=pairs, N=F, K=W, y=a, lda=W, ldy=F, batch=E, stride_w=F * W, act=self.act,
+                       a_rows=tok_of, z_start=z_start)
+        y = torch.empty(pairs, W, dtype=torch.float32, device=h.device)
+        seq_ops.linear(a, self.w_down, M=pairs, N=W, K=F, y=y, lda=F, ldy=W, batch=E, stride_w=W * F, z_start=z_start)
+        seq_ops.moe_combine(y, where, wts, x)
+
+
+class TokenSide(nn.Module):
+    """Per-layer token input: e = this layer's slice of a second embedding table at the token,
+    y = W_proj (gelu_tanh(W_gate x) * e), x <- x + y / rms(y) * w (plain weight). Reads the stream after the
+    layer's feed-forward; a looped layer uses the same slice in every pass."""
+
+    def __init__(self, layer: int, dim: int, table: torch.Tensor, w: Dict[str, torch.Tensor], eps: float, device,
+                 dtype) -> None:
+        super().__init__()
+        self.col0, self.dim, self.eps = layer * dim, dim, eps
+        self.table = table  # shared by all layers (owned by the model)
+        self.register_buffer("w_gate", w["gate"].to(device=device, dtype=dtype).contiguous())
+        self.register_buffer("w_proj", w["proj"].to(device=device, dtype=dtype).contiguous())
+        self.register_buffer("norm_w", _f32(w["norm"], device))
+
+    def forward(self, x: torch.Tensor, tokens: torch.Tensor) -> None:
+        seq_ops.token_side(x, tokens, self.table, self.col0, self.w_gate, self.w_proj, self.norm_w, self.eps)
+
+
+MIXERS = {"retention": Retention, "latent_attention": LatentAttention}

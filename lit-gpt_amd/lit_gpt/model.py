@@ -617,6 +617,60 @@ class KVCache(nn.Module):
         torch.nn.init.zeros_(self.v)
 
 
+class RetentionState(nn.Module):
+    """Per-slot recurrent state of a retention mixer: (slots, heads, key dim, value dim) fp32. A slot belongs to one
+    sequence at a time; the kernel starts a sequence at position 0 from zeros, so a slot that is given out again
+    needs no clearing. One instance per layer run (a looped layer has one per pass)."""
+
+    def __init__(self, slots: int, heads: int, dim: int, vdim: int, device: Optional[torch.device] = None) -> None:
+        super().__init__()
+        self.register_buffer("s", torch.zeros(slots, heads, dim, vdim, device=device, dtype=torch.float32),
+                             persistent=False)
+
+    @property
+    def slots(self) -> int:
+        return self.s.size(0)
+
+    def grow(self, slots: int) -> None:
+        if slots > self.slots:
+            s = torch.zeros(slots, *self.s.shape[1:], device=self.s.device, dtype=torch.float32)
+            s[: self.slots] = self.s
+            self.s = s
+
+    def reset_parameters(self) -> None:
+        torch.nn.init.zeros_(self.s)
+
+
+class LatentKVCache(nn.Module):
+    """Cache of a latent-attention mixer: per slot and position the normed latent ``c`` (kv_rank values, in the
+    compute dtype) and the rotated key part shared by all heads (``kr``, fp32). Keys and values are never stored
+    per head: the attention kernel works in the latent space. One instance per layer run."""
+
+    def __init__(self, slots: int, max_seq_length: int, kv_rank: int, rot_dim: int,
+                 device: Optional[torch.device] = None, dtype: Optional[torch.dtype] = None) -> None:
+        super().__init__()
+        self.register_buffer("c", torch.zeros(slots, max_seq_length, kv_rank, device=device,
+                                              dtype=dtype or torch.bfloat16), persistent=False)
+        self.register_buffer("kr", torch.zeros(slots, max_seq_length, rot_dim, device=device, dtype=torch.float32),
+                             persistent=False)
+
+    @property
+    def slots(self) -> int:
+        return self.c.size(0)
+
+    def grow(self, slots: int) -> None:
+        if slots > self.slots:
+            for name in ("c", "kr"):
+                old = getattr(self, name)
+                new = torch.zeros(slots, *old.shape[1:], device=old.device, dtype=old.dtype)
+                new[: old.size(0)] = old
+                setattr(self, name, new)
+
+    def reset_parameters(self) -> None:
+        torch.nn.init.zeros_(self.c)
+        torch.nn.init.zeros_(self.kr)
+
+
 def build_rope_cache(seq_len: int, n_elem: int, device: Optional[torch.device] = None, base: int = 10000,
                      condense_ratio: int = 1) -> Tuple[torch.Tensor, torch.Tensor]:
     """cos/sin tables (seq_len, n_elem) in fp32 (model.py:746-764).

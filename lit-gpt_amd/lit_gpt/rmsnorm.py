@@ -28,3 +28,21 @@ class RMSNorm(nn.Module):
 
     def reset_parameters(self) -> None:
         torch.nn.init.ones_(self.weight)
+
+
+class StreamRMSNorm(nn.Module):
+    """RMS norm over rows of the fp32 residual stream (``lgs_rmsnorm``): x / sqrt(mean(x^2) + eps) * (offset + w).
+    ``offset`` 1.0 serves checkpoints whose norm weight is stored around zero, 0.0 the plain weight; the weight is
+    kept in fp32 whatever the model's compute dtype."""
+
+    def __init__(self, size: int, eps: float = 1e-5, offset: float = 0.0) -> None:
+        super().__init__()
+        self.register_buffer("weight", torch.zeros(size) if offset else torch.ones(size))
+        self.eps, self.offset = eps, offset
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        from lit_gpt import seq_ops
+
+        if not x.is_cuda:
+            _gpu_only("StreamRMSNorm")
+        return seq_ops.rmsnorm(x, self.weight, offset=self.offset, eps=self.eps)

@@ -1,0 +1,279 @@
+"""Python view of ``liblitgpt_seq.so`` (declared in ``include/litgpt_seq.h``): the kernels of the layered models.
+
+Same conventions as ``lit_gpt.ops``: thin wrappers that check device / dtype / contiguity, pass raw device pointers,
+launch on torch's current HIP stream (capturable into a HIP graph) and raise on a non-zero return code. There is
+no CPU path. Activations are fp32; a weight is a bf16 or an fp32 tensor and its dtype picks the kernel: bf16 weights
+take the activation rounded to bf16 with fp32 sums (MFMA tiles, streaming GEMVs), fp32 weights run plain fp32 FMA.
+
+The library is separate from ``liblitgpt_amd.so`` so that serving a layered model compiles four small sources only;
+``build_library`` runs that ``make`` target when the library is missing.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+from pathlib import Path
+from typing import Optional
+
+import torch
+
+from lit_gpt.ops import NativeLibraryError, _dev, _opt, _stream
+
+LIB_PATH = Path(os.environ.get("LGS_LIB", Path(__file__).resolve().parent / "_lib" / "liblitgpt_seq.so"))
+CSRC = Path(__file__).resolve().parent.parent / "csrc"
+
+ACT_NONE, ACT_RELU2, ACT_GELU_TANH, ACT_SILU, ACT_SIGMOID = 0, 1, 2, 3, 4
+
+_P, _I, _L, _F = ctypes.c_void_p, ctypes.c_int, ctypes.c_long, ctypes.c_float
+
+SIGNATURES = {
+    "lgs_version": [],
+    "lgs_last_error_string": [],
+    "lgs_linear": [_P, _L, _L, _P, _I, _L, _P, _L, _L, _I, _I, _I, _I, _I, _I, _P, _P, _P],
+    "lgs_embed": [_P, _P, _I, _F, _P, _I, _I, _I, _P],
+    "lgs_rmsnorm": [_P, _L, _P, _F, _F, _P, _L, _I, _I, _I, _P],
+    "lgs_gather_rows": [_P, _P, _P, _I, _I, _P],
+    "lgs_retention": [_P, _P, _P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _P],
+    "lgs_head_gate": [_P, _P, _L, _I, _I, _I, _I, _F, _I, _P],
+    "lgs_latent_prepare": [_P, _L, _I, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P],
+    "lgs_latent_attention": [_P, _P, _L, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P],
+    "lgs_glu": [_P, _P, _L, _P, _I, _I, _I, _P],
+    "lgs_moe_route": [_P, _L, _I, _I, _I, _P, _P, _P],
+    "lgs_moe_up": [_P, _L, _P, _I, _P, _P, _I, _I, _I, _I, _I, _P],
+    "lgs_moe_down": [_P, _P, _I, _P, _P, _P, _L, _I, _I, _I, _I, _P],
+    "lgs_moe_sort": [_P, _I, _I, _I, _P, _P, _P, _P],
+    "lgs_moe_combine": [_P, _P, _P, _P, _L, _I, _I, _I, _P],
+    "lgs_token_side": [_P, _P, _P, _I, _L, _I, _P, _P, _P, _I, _I, _I, _I, _F, _P],
+}
+_RESTYPES = {"lgs_last_error_string": ctypes.c_char_p}
+
+_lib: Optional[ctypes.CDLL] = None
+
+
+def build_library() -> Path:
+    """Compile the library in-tree (``make seq``: hipcc --offload-arch=gfx950) unless it is there already."""
+    if not LIB_PATH.is_file():
+        jobs = str(min(16, os.cpu_count() or 8))
+        subprocess.run(["make", "-C", str(CSRC), f"-j{jobs}", "seq"], check=True, stdout=subprocess.DEVNULL)
+    return LIB_PATH
+
+
+def load_library() -> ctypes.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not LIB_PATH.is_file():
+        raise NativeLibraryError(f"HIP library not found at {LIB_PATH}. Build it with `make -C lit-gpt_amd/csrc seq` "
+                                 "(hipcc --offload-arch=gfx950). There is no CPU fallback.")
+    lib = ctypes.CDLL(str(LIB_PATH))
+    for name, argtypes in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.argtypes = argtypes
+        fn.restype = _RESTYPES.get(name, ctypes.c_int)
+    _lib = lib
+    return lib
+
+
+def _check(rc: int) -> None:
+    if rc != 0:
+        msg = load_library().lgs_last_error_string()
+        raise RuntimeError(f"liblitgpt_seq error {rc}: {msg.decode() if msg else ''}")
+
+
+def _wf32(w: torch.Tensor, name: str) -> int:
+    if w.dtype not in (torch.bfloat16, torch.float32):
+        raise TypeError(f"{name}: weights are bf16 or fp32, got {w.dtype}")
+    return int(w.dtype == torch.float32)
+
+
+F32, I32 = torch.float32, torch.int32
+
+
+def linear(a: torch.Tensor, w: torch.Tensor, *, M: int, N: int, K: int, y: torch.Tensor, a_off: int = 0, lda: int,
+           y_off: int = 0, ldy: int, batch: int = 1, stride_a: int = 0, stride_w: int = 0, stride_y: int = 0,
+           accumulate: bool = False, act: int = ACT_NONE, a_rows: Optional[torch.Tensor] = None,
+           z_start: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """y[z] (+)= act(a[z] w[z]^T) over ``batch`` strided operands; offsets and strides count elements. With
+    ``z_start`` (batch + 1 int32 row bounds) batch z owns that range of a row list of at most M rows, whose A rows
+    are ``a_rows`` (or the list places themselves) and whose Y rows are the list places."""
+    ap = _dev(a, "a", F32) + 4 * a_off
+    yp = _dev(y, "y", F32) + 4 * y_off
+    need_a = a_off + (batch - 1) * stride_a + (0 if a_rows is not None else (M - 1) * lda) + K
+    need_y = y_off + (batch - 1) * stride_y * (0 if z_start is not None else 1) + (M - 1) * ldy + N
+    if a.numel() < need_a or y.numel() < need_y or w.numel() < (batch - 1) * stride_w + N * K:
+        raise ValueError("linear: an operand is smaller than the sizes and strides say")
+    _check(load_library().lgs_linear(ap, lda, stride_a, _dev(w, "w"), _wf32(w, "w"), stride_w, yp, ldy, stride_y,
+                                     M, N, K, batch, int(accumulate), act, _opt(a_rows, "a_rows", I32),
+                                     _opt(z_start, "z_start", I32), _stream()))
+    return y
+
+
+def embed(tokens: torch.Tensor, table: torch.Tensor, scale: float) -> torch.Tensor:
+    T, (V, W) = tokens.numel(), table.shape
+    x = torch.empty(T, W, dtype=F32, device=tokens.device)
+    _check(load_library().lgs_embed(_dev(tokens, "tokens", I32), _dev(table, "table"), _wf32(table, "table"),
+                                    float(scale), x.data_ptr(), T, W, V, _stream()))
+    return x
+
+
+def rmsnorm(x: torch.Tensor, weight: Optional[torch.Tensor], *, offset: float, eps: float,
+            out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Rows of a contiguous (rows, n) tensor: x / sqrt(mean(x^2) + eps) * (offset + weight) (no weight: unit RMS)."""
+    rows, n = x.shape
+    y = out if out is not None else torch.empty_like(x)
+    if weight is not None and weight.numel() != n:
+        raise ValueError("rmsnorm: weight size")
+    _check(load_library().lgs_rmsnorm(_dev(x, "x", F32), n, _opt(weight, "weight", F32), float(offset), float(eps),
+                                      _dev(y, "y", F32), n, rows, 1, n, _stream()))
+    return y
+
+
+def gather_rows(x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
+    y = torch.empty(rows.numel(), x.shape[1], dtype=F32, device=x.device)
+    _check(load_library().lgs_gather_rows(_dev(x, "x", F32), _dev(rows, "rows", I32), y.data_ptr(), rows.numel(),
+                                          x.shape[1], _stream()))
+    return y
+
+
+def retention(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, state: torch.Tensor, decay: torch.Tensor,
+              inv_freq: Optional[torch.Tensor], seq_start: torch.Tensor, seq_slot: torch.Tensor,
+              seq_pos0: torch.Tensor, *, H: int, d: int, dv: int, rot_dims: int, k_scale: float) -> torch.Tensor:
+    """proj (T, ld) holds q, k (H * d each) and v (H * dv) at the given column offsets; state (slots, H, d, dv) fp32
+    is read (unless a sequence starts at position 0) and left at the step's last token. Returns o (T, H * dv)."""
+    T, ld = proj.shape
+    B = seq_slot.numel()
+    if tuple(state.shape[1:]) != (H, d, dv) or seq_start.numel() != B + 1 or decay.numel() != H:
+        raise ValueError("retention: state / sequence table shapes")
+    if max(q_off, k_off) + H * d > ld or v_off + H * dv > ld:
+        raise ValueError("retention: projections outside the row")
+    out = torch.empty(T, H * dv, dtype=F32, device=proj.device)
+    base = _dev(proj, "proj", F32)
+    _check(load_library().lgs_retention(base + 4 * q_off, base + 4 * k_off, base + 4 * v_off, ld,
+                                        _dev(state, "state", F32), _dev(decay, "decay", F32),
+                                        _opt(inv_freq, "inv_freq", F32), _dev(seq_start, "seq_start", I32),
+                                        _dev(seq_slot, "seq_slot", I32), _dev(seq_pos0, "seq_pos0", I32),
+                                        out.data_ptr(), B, H, d, dv, rot_dims, float(k_scale), _stream()))
+    return out
+
+
+def head_gate(o: torch.Tensor, proj: torch.Tensor, g_off: int, *, H: int, dv: int, unit_norm: bool, eps: float,
+              act: int) -> torch.Tensor:
+    """In place on o (T, H * dv): per head optional unit RMS, then times act(gate), the gate at proj[:, g_off:]."""
+    T, ld = proj.shape
+    if o.shape != (T, H * dv) or g_off + H * dv > ld:
+        raise ValueError("head_gate: shapes")
+    _check(load_library().lgs_head_gate(_dev(o, "o", F32), _dev(proj, "proj", F32) + 4 * g_off, ld, T, H, dv,
+                                        int(unit_norm), float(eps), act, _stream()))
+    return o
+
+
+def latent_prepare(proj: torch.Tensor, q_off: int, kv_off: int, cache_c: torch.Tensor, cache_kr: torch.Tensor,
+                   norm_w: torch.Tensor, inv_freq: Optional[torch.Tensor], slot: torch.Tensor, pos: torch.Tensor, *,
+                   H: int, d: int, dr: int, r: int, rot_dims: int, eps: float) -> None:
+    T, ld = proj.shape
+    slots, S = cache_c.shape[:2]
+    if tuple(cache_c.shape) != (slots, S, r) or tuple(cache_kr.shape) != (slots, S, dr) or norm_w.numel() != r:
+        raise ValueError("latent_prepare: cache shapes")
+    if q_off + H * (d + dr) > ld or kv_off + r + dr > ld or slot.numel() != T or pos.numel() != T:
+        raise ValueError("latent_prepare: projections outside the row")
+    _check(load_library().lgs_latent_prepare(_dev(proj, "proj", F32), ld, q_off, kv_off, _dev(cache_c, "cache_c"),
+                                             _wf32(cache_c, "cache_c"), _dev(cache_kr, "cache_kr", F32),
+                                             _dev(norm_w, "norm_w", F32), _opt(inv_freq, "inv_freq", F32),
+                                             _dev(slot, "slot", I32), _dev(pos, "pos", I32), T, H, d, dr, r, rot_dims,
+                                             S, float(eps), _stream()))
+
+
+def latent_attention(qc: torch.Tensor, proj: torch.Tensor, q_off: int, cache_c: torch.Tensor, cache_kr: torch.Tensor,
+                     sink: Optional[torch.Tensor], slot: torch.Tensor, pos: torch.Tensor, *, H: int, d: int, dr: int,
+                     r: int, scale: float) -> torch.Tensor:
+    T, ld = proj.shape
+    S = cache_c.shape[1]
+    if qc.shape != (T, H * r) or (sink is not None and sink.numel() != H):
+        raise ValueError("latent_attention: shapes")
+    out = torch.empty(T, H * r, dtype=F32, device=proj.device)
+    _check(load_library().lgs_latent_attention(_dev(qc, "qc", F32), _dev(proj, "proj", F32), ld, q_off,
+                                               _dev(cache_c, "cache_c"), _wf32(cache_c, "cache_c"),
+                                               _dev(cache_kr, "cache_kr", F32), _opt(sink, "sink", F32),
+                                               _dev(slot, "slot", I32), _dev(pos, "pos", I32), out.data_ptr(), T, H,
+                                               d, dr, r, S, float(scale), _stream()))
+    return out
+
+
+def glu(proj: torch.Tensor, a_off: int, b_off: int, n: int, act: int) -> torch.Tensor:
+    T, ld = proj.shape
+    if max(a_off, b_off) + n > ld:
+        raise ValueError("glu: columns outside the row")
+    out = torch.empty(T, n, dtype=F32, device=proj.device)
+    base = _dev(proj, "proj", F32)
+    _check(load_library().lgs_glu(base + 4 * a_off, base + 4 * b_off, ld, out.data_ptr(), T, n, act, _stream()))
+    return out
+
+
+def moe_route(proj: torch.Tensor, z_off: int, E: int, top: int):
+    T, ld = proj.shape
+    if z_off + E > ld:
+        raise ValueError("moe_route: router logits outside the row")
+    ids = torch.empty(T, top, dtype=I32, device=proj.device)
+    wts = torch.empty(T, top, dtype=F32, device=proj.device)
+    _check(load_library().lgs_moe_route(_dev(proj, "proj", F32) + 4 * z_off, ld, T, E, top, ids.data_ptr(),
+                                        wts.data_ptr(), _stream()))
+    return ids, wts
+
+
+def moe_up(h: torch.Tensor, up: torch.Tensor, ids: torch.Tensor, act: int) -> torch.Tensor:
+    T, K = h.shape
+    E, F, K2 = up.shape
+    top = ids.shape[1]
+    if K2 != K or ids.shape[0] != T:
+        raise ValueError("moe_up: shapes")
+    buf = torch.empty(T * top, F, dtype=F32, device=h.device)
+    _check(load_library().lgs_moe_up(_dev(h, "h", F32), K, _dev(up, "up"), _wf32(up, "up"), _dev(ids, "ids", I32),
+                                     buf.data_ptr(), T, top, F, K, act, _stream()))
+    return buf
+
+
+def moe_down(actbuf: torch.Tensor, down: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, x: torch.Tensor) -> None:
+    T, top = ids.shape
+    E, N, F = down.shape
+    if actbuf.shape != (T * top, F) or x.shape != (T, N):
+        raise ValueError("moe_down: shapes")
+    _check(load_library().lgs_moe_down(_dev(actbuf, "actbuf", F32), _dev(down, "down"), _wf32(down, "down"),
+                                       _dev(ids, "ids", I32), _dev(wts, "wts", F32), _dev(x, "x", F32), N, T, top, N,
+                                       F, _stream()))
+
+
+def moe_sort(ids: torch.Tensor, E: int):
+    T, top = ids.shape
+    dev = ids.device
+    z_start = torch.empty(E + 1, dtype=I32, device=dev)
+    tok_of = torch.empty(T * top, dtype=I32, device=dev)
+    where = torch.empty(T * top, dtype=I32, device=dev)
+    _check(load_library().lgs_moe_sort(_dev(ids, "ids", I32), T * top, top, E, z_start.data_ptr(), tok_of.data_ptr(),
+                                       where.data_ptr(), _stream()))
+    return z_start, tok_of, where
+
+
+def moe_combine(y: torch.Tensor, where: torch.Tensor, wts: torch.Tensor, x: torch.Tensor) -> None:
+    T, top = wts.shape
+    N = x.shape[1]
+    if y.shape != (T * top, N) or where.numel() != T * top:
+        raise ValueError("moe_combine: shapes")
+    _check(load_library().lgs_moe_combine(_dev(y, "y", F32), _dev(where, "where", I32), _dev(wts, "wts", F32),
+                                          _dev(x, "x", F32), N, T, top, N, _stream()))
+
+
+def token_side(x: torch.Tensor, tokens: torch.Tensor, table: torch.Tensor, col0: int, gate_w: torch.Tensor,
+               proj_w: torch.Tensor, norm_w: torch.Tensor, eps: float) -> None:
+    T, W = x.shape
+    dim = gate_w.shape[0]
+    V, ld = table.shape
+    if gate_w.shape != (dim, W) or proj_w.shape != (W, dim) or norm_w.numel() != W or col0 + dim > ld:
+        raise ValueError("token_side: shapes")
+    if len({table.dtype, gate_w.dtype, proj_w.dtype}) != 1:
+        raise TypeError("token_side: weights of one dtype expected")
+    _check(load_library().lgs_token_side(_dev(x, "x", F32), _dev(tokens, "tokens", I32), _dev(table, "table"),
+                                         _wf32(table, "table"), ld, col0, _dev(gate_w, "gate_w"),
+                                         _dev(proj_w, "proj_w"), _dev(norm_w, "norm_w", F32), T, W, dim, V,
+                                         float(eps), _stream()))

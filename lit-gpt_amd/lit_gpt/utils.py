@@ -35,3 +35,35 @@ def check_valid_checkpoint_dir(checkpoint_dir: Path) -> None:
 def get_default_supported_precision(training: bool) -> str:
     """bf16 on MI355X (reference lit_gpt/utils.py:334-347 picks bf16 when the device supports it)."""
     return "bf16-mixed" if training else "bf16-true"
+
+
+def read_safetensors(path) -> dict:
+    """{name: tensor} of a .safetensors file: an 8-byte little-endian header length, that many bytes of JSON
+    (name -> dtype, shape, data_offsets), then the raw little-endian data. Nothing in the file is executed."""
+    import json
+    import struct
+
+    import numpy as np
+    import torch
+
+    kinds = {"BF16": (torch.bfloat16, 2), "F16": (torch.float16, 2), "F32": (torch.float32, 4),
+             "F64": (torch.float64, 8), "I32": (torch.int32, 4), "I64": (torch.int64, 8), "U8": (torch.uint8, 1),
+             "I8": (torch.int8, 1), "I16": (torch.int16, 2), "BOOL": (torch.bool, 1)}
+    with open(path, "rb") as f:
+        (n,) = struct.unpack("<Q", f.read(8))
+        header = json.loads(f.read(n))
+    data = np.memmap(path, dtype=np.uint8, mode="r", offset=8 + n)
+    out = {}
+    for name, meta in header.items():
+        if name == "__metadata__":
+            continue
+        dtype, size = kinds[meta["dtype"]]
+        lo, hi = meta["data_offsets"]
+        count = 1
+        for s in meta["shape"]:
+            count *= int(s)
+        if hi - lo != count * size:
+            raise ValueError(f"{path}: tensor {name!r} has {hi - lo} bytes for shape {meta['shape']}")
+        raw = torch.from_numpy(np.array(data[lo:hi]))  # a private copy: the map is read-only
+        out[name] = raw.view(dtype).reshape(meta["shape"]) if count else torch.empty(meta["shape"], dtype=dtype)
+    return out
