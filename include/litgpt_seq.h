@@ -1,0 +1,97 @@
+/*
+ * litgpt_seq.h — C ABI of liblitgpt_seq.so: the MI355X (gfx950) kernels of the layered models (retention and
+ * latent-attention mixers, gated and sparse feed-forwards, per-layer token inputs) over an fp32 residual stream.
+ *
+ * Conventions: plain device pointers and sizes; every buffer is caller-owned; launches are asynchronous on `stream`
+ * (graph-capturable); 0 on success, otherwise a hipError_t value with a message from lgs_last_error_string()
+ * (thread-local). Activations are fp32. A weight matrix is [out][in], bf16 (w_f32 = 0: the activation operand is
+ * rounded to bf16, sums are fp32) or fp32 (w_f32 = 1: plain fp32). Offsets and strides count elements.
+ * A step is a packed batch: per token an int32 cache slot and position; per sequence its first row (seq_start,
+ * B + 1 entries), slot and first position.
+ */
+#ifndef LITGPT_SEQ_H
+#define LITGPT_SEQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ihipStream_t* lgs_stream_t; /* == hipStream_t */
+
+/* activations (lgs_linear epilogue, lgs_glu, lgs_head_gate, lgs_moe_up) */
+#define LGS_ACT_NONE 0
+#define LGS_ACT_RELU2 1     /* max(z, 0)^2 */
+#define LGS_ACT_GELU_TANH 2 /* 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))) */
+#define LGS_ACT_SILU 3
+#define LGS_ACT_SIGMOID 4
+
+const char* lgs_last_error_string(void);
+int lgs_version(void);
+
+/* y[z] (+)= act(a[z] w[z]^T) for z < batch: a[z] = a + z stride_a (M rows of K, row stride lda), w[z] = w + z stride_w
+ * ([N][K]), y[z] = y + z stride_y (row stride ldy). M <= 8: streaming GEMV; otherwise 128x128 MFMA tiles (bf16) or
+ * 64x64 FMA tiles (fp32). z_start (batch + 1 bounds, device) makes it grouped: batch z owns rows
+ * [z_start[z], z_start[z+1]) of a list of at most M rows; list row i reads A row a_rows[i] (or i) and writes Y row i
+ * (stride_a and stride_y are then ignored for the rows' place). */
+int lgs_linear(const float* a, long lda, long stride_a, const void* w, int w_f32, long stride_w, float* y, long ldy,
+               long stride_y, int M, int N, int K, int batch, int accumulate, int act, const int* a_rows,
+               const int* z_start, lgs_stream_t stream);
+/* x[t] = table[tokens[t]] * scale */
+int lgs_embed(const int* tokens, const void* table, int w_f32, float scale, float* x, int T, int W, int vocab,
+              lgs_stream_t stream);
+/* group g of row r: y = x / sqrt(mean(x^2) + eps) * (offset + weight) (weight NULL: unit RMS), n values per group */
+int lgs_rmsnorm(const float* x, long ldx, const float* weight, float offset, float eps, float* y, long ldy, int rows,
+                int groups, int n, lgs_stream_t stream);
+int lgs_gather_rows(const float* x, const int* rows, float* y, int n_rows, int W, lgs_stream_t stream);
+
+/* retention: rotary (pairs i, i + rot_dims/2; angle = position * inv_freq[i]) on q and k, k * k_scale, then per
+ * sequence and head S <- decay S + k v^T, o = S^T q. state [slots][H][d][dv] fp32 is read unless the sequence's
+ * first position is 0 and written back at the end of the step. d <= 256. */
+int lgs_retention(const float* q, const float* k, const float* v, long ld, float* state, const float* decay,
+                  const float* inv_freq, const int* seq_start, const int* seq_slot, const int* seq_pos0, float* out,
+                  int B, int H, int d, int dv, int rot_dims, float k_scale, lgs_stream_t stream);
+/* in place on o [T][H][dv]: (unit_norm ? o / rms(o) per head : o) * act(g[t * ldg + h * dv + i]) */
+int lgs_head_gate(float* o, const float* g, long ldg, int T, int H, int dv, int unit_norm, float eps, int act,
+                  lgs_stream_t stream);
+/* latent attention, per token: c = rmsnorm(proj[kv_off .. + r]) * norm_w -> cache_c[slot][pos] (bf16, or fp32 with
+ * cache_f32); rotary (pairs 2i, 2i + 1) of proj[kv_off + r .. + dr] -> cache_kr[slot][pos] (fp32); the rotated
+ * part of every head's query (at q_off + h (d + dr) + d) is rotated in place. */
+int lgs_latent_prepare(float* proj, long ld, int q_off, int kv_off, void* cache_c, int cache_f32, float* cache_kr,
+                       const float* norm_w, const float* inv_freq, const int* slot, const int* pos, int T, int H,
+                       int d, int dr, int r, int rot_dims, int max_seq, float eps, lgs_stream_t stream);
+/* out[t][h] = sum_j p_j c_j over cached rows j <= pos[t] of slot[t], p = softmax over
+ * (qc[t][h] . c_j + q_rot[t][h] . kr_j) * scale with exp(sink[h]) added to the denominator (sink NULL: none).
+ * r <= 512, dr <= 128. */
+int lgs_latent_attention(const float* qc, const float* proj, long ld, int q_off, const void* cache_c, int cache_f32,
+                         const float* cache_kr, const float* sink, const int* slot, const int* pos, float* out, int T,
+                         int H, int d, int dr, int r, int max_seq, float scale, lgs_stream_t stream);
+
+/* out[t][i] = act(a[t * ld + i]) * b[t * ld + i], i < n */
+int lgs_glu(const float* a, const float* b, long ld, float* out, int T, int n, int act, lgs_stream_t stream);
+/* per token: ids / wts [T][top] = the top largest of z[t * ld .. + E] (lowest index first among equals) and the
+ * softmax over those. E <= 256. */
+int lgs_moe_route(const float* z, long ld, int T, int E, int top, int* ids, float* wts, lgs_stream_t stream);
+/* streaming experts: actbuf[t * top + k] = act(up[ids[t][k]] h[t]); x[t] += sum_k wts[t][k] down[ids[t][k]] actbuf[..] */
+int lgs_moe_up(const float* h, long ldh, const void* up, int w_f32, const int* ids, float* actbuf, int T, int top,
+               int F, int K, int act, lgs_stream_t stream);
+int lgs_moe_down(const float* actbuf, const void* down, int w_f32, const int* ids, const float* wts, float* x,
+                 long ldx, int T, int top, int N, int F, lgs_stream_t stream);
+/* stable counting sort of the (token, choice) pairs by expert: z_start [E + 1], tok_of [pairs] (token of each sorted
+ * entry), where [pairs] (sorted place of each pair) */
+int lgs_moe_sort(const int* ids, int pairs, int top, int E, int* z_start, int* tok_of, int* where,
+                 lgs_stream_t stream);
+/* x[t] += sum_k wts[t][k] * y[where[t * top + k]] */
+int lgs_moe_combine(const float* y, const int* where, const float* wts, float* x, long ldx, int T, int top, int N,
+                    lgs_stream_t stream);
+/* x[t] += unit_rms(proj_w (gelu_tanh(gate_w x[t]) * table[tokens[t]][col0 .. + dim])) * norm_w */
+int lgs_token_side(float* x, const int* tokens, const void* table, int w_f32, long ld_table, int col0,
+                   const void* gate_w, const void* proj_w, const float* norm_w, int T, int W, int dim, int vocab,
+                   float eps, lgs_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

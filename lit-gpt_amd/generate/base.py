@@ -108,7 +108,8 @@ def generate(model: GPT, prompt: torch.Tensor, max_returned_tokens: int, *, temp
     n_steps = max_returned_tokens - T - 1
     if n_steps <= 0:
         return torch.cat(tokens)
-    if use_graph and graph_sampling(model, temperature, top_k):
+    # (a model class may opt out of the captured step with ``decode_graph = False``: it is then stepped eagerly)
+    if use_graph and getattr(model, "decode_graph", True) and graph_sampling(model, temperature, top_k):
         from lit_gpt.runtime import DecodeGraph
 
         # (the prefill's token is never tested against eos: the reference's loop only tests the decoded ones,
