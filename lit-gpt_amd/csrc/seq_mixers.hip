@@ -96,6 +96,145 @@ __global__ void __launch_bounds__(256) retention_scan_kernel(RetArgs p) {
   }
 }
 
+// The prompt form: the same recurrence over chunks of 64 tokens as fp32 matrix products (v_mfma_f32_16x16x4_f32).
+// With S the state at the chunk's start, n its token count and i, j local positions:
+//   o_i = decay^(i+1) S^T q_i + sum_{j <= i} decay^(i-j) (q_i . k_j) v_j,   S' = decay^n S + sum_j decay^(n-1-j) k_j v_j^T
+// grid (B, H, ceil(dv / 64)); a workgroup keeps 64 columns of the state in LDS and walks its sequence's chunks.
+// LDS (floats): Q, K [64][DP], V [64][80], scores [64][66], S [DPAD][80], powers of the decay [66]; d <= 128.
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+constexpr int kRC = 64, kVS = 80, kAS = 66;
+
+__global__ void __launch_bounds__(256) retention_chunk_kernel(RetArgs p) {
+  extern __shared__ float lds[];
+  const int b = blockIdx.x, h = blockIdx.y, col0 = blockIdx.z * 64;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int d = p.d, dv = p.dv, half = p.rot_dims / 2;
+  const int DT = (d + 15) / 16, DPAD = DT * 16, DP = DPAD + 2;
+  float* Qs = lds;
+  float* Ks = Qs + kRC * DP;
+  float* Vs = Ks + kRC * DP;
+  float* As = Vs + kRC * kVS;
+  float* Ss = As + kRC * kAS;
+  float* pw = Ss + DPAD * kVS;
+  const int t0 = p.seq_start[b], t1 = p.seq_start[b + 1];
+  const int pos0 = p.seq_pos0[b];
+  const float lam = p.decay[h];
+  float* sp = p.state + (((size_t)p.seq_slot[b] * p.H + h) * d) * dv;
+  for (int i = tid; i < DPAD * 64; i += 256) {
+    const int row = i >> 6, c = i & 63;
+    Ss[row * kVS + c] = (pos0 > 0 && row < d && col0 + c < dv) ? sp[(size_t)row * dv + col0 + c] : 0.0f;
+  }
+  if (tid <= 64) pw[tid] = powf(lam, (float)tid);
+  const int fr = lane & 15, fk = lane >> 4;
+  for (int tc = t0; tc < t1; tc += kRC) {
+    const int n = min(kRC, t1 - tc);
+    // ---- load: q and k rotated (pairs dd, dd + half), k scaled; rows past n and dims past d are zero
+    for (int i = tid; i < kRC * DPAD; i += 256) {
+      const int row = i / DPAD, dd = i - row * DPAD;
+      if (dd >= half && dd < 2 * half) continue;  // written by its partner
+      const bool in = row < n && dd < d;
+      const float* qr = p.q + (size_t)(tc + row) * p.ld + (size_t)h * d;
+      const float* kr = p.k + (size_t)(tc + row) * p.ld + (size_t)h * d;
+      if (dd < half) {
+        float q0 = 0.f, q1 = 0.f, k0 = 0.f, k1 = 0.f;
+        if (row < n) {
+          float sn, cs;
+          sincosf((float)(pos0 + (tc - t0) + row) * p.inv_freq[dd], &sn, &cs);
+          const float qu = qr[dd], qv = qr[dd + half], ku = kr[dd], kv = kr[dd + half];
+          q0 = qu * cs - qv * sn;
+          q1 = qv * cs + qu * sn;
+          k0 = (ku * cs - kv * sn) * p.k_scale;
+          k1 = (kv * cs + ku * sn) * p.k_scale;
+        }
+        Qs[row * DP + dd] = q0;
+        Qs[row * DP + dd + half] = q1;
+        Ks[row * DP + dd] = k0;
+        Ks[row * DP + dd + half] = k1;
+      } else {
+        Qs[row * DP + dd] = in ? qr[dd] : 0.0f;
+        Ks[row * DP + dd] = in ? kr[dd] * p.k_scale : 0.0f;
+      }
+    }
+    for (int i = tid; i < kRC * 64; i += 256) {
+      const int row = i >> 6, c = i & 63;
+      Vs[row * kVS + c] = (row < n && col0 + c < dv) ? p.v[(size_t)(tc + row) * p.ld + (size_t)h * dv + col0 + c] : 0.0f;
+    }
+    __syncthreads();
+    // ---- wave w owns tokens 16 w .. 16 w + 15: decayed causal scores, and the carried state's share of o
+    const int ti = wave;
+    for (int tj = 0; tj < 4; ++tj) {
+      f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+      if (tj <= ti)
+        for (int k = 0; k < DPAD; k += 4)
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(Qs[(ti * 16 + fr) * DP + k + fk], Ks[(tj * 16 + fr) * DP + k + fk],
+                                                     acc, 0, 0, 0);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int i = ti * 16 + fk * 4 + r, j = tj * 16 + fr;
+        As[i * kAS + j] = j <= i ? acc[r] * pw[i - j] : 0.0f;
+      }
+    }
+    f32x4_t o[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) o[c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int k = 0; k < DPAD; k += 4) {
+      const float a = Qs[(ti * 16 + fr) * DP + k + fk];
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        o[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, Ss[(k + fk) * kVS + c * 16 + fr], o[c], 0, 0, 0);
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o[c][r] *= pw[ti * 16 + fk * 4 + r + 1];
+    __syncthreads();
+    // ---- o += scores . V (keys up to the wave's last token), then out
+    for (int k = 0; k < (ti + 1) * 16; k += 4) {
+      const float a = As[(ti * 16 + fr) * kAS + k + fk];
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        o[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, Vs[(k + fk) * kVS + c * 16 + fr], o[c], 0, 0, 0);
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int i = ti * 16 + fk * 4 + r, col = col0 + c * 16 + fr;
+        if (i < n && col < dv) p.out[(size_t)(tc + i) * p.H * dv + (size_t)h * dv + col] = o[c][r];
+      }
+    // ---- state: S' = decay^n S + sum_j decay^(n-1-j) k_j v_j^T; each element of S belongs to one lane
+    const float pn = pw[n];
+    for (int td = wave; td < DT; td += 4) {
+      f32x4_t s[4];
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) s[c][r] = pn * Ss[(td * 16 + fk * 4 + r) * kVS + c * 16 + fr];
+      for (int k = 0; k < kRC; k += 4) {
+        const int j = k + fk;
+        const float a = j < n ? Ks[j * DP + td * 16 + fr] * pw[n - 1 - j] : 0.0f;
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          s[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, Vs[j * kVS + c * 16 + fr], s[c], 0, 0, 0);
+      }
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) Ss[(td * 16 + fk * 4 + r) * kVS + c * 16 + fr] = s[c][r];
+    }
+    __syncthreads();
+  }
+  for (int i = tid; i < DPAD * 64; i += 256) {
+    const int row = i >> 6, c = i & 63;
+    if (row < d && col0 + c < dv) sp[(size_t)row * dv + col0 + c] = Ss[row * kVS + c];
+  }
+}
+
+static size_t retention_chunk_lds(int d) {
+  const int DPAD = (d + 15) / 16 * 16, DP = DPAD + 2;
+  return (size_t)(2 * kRC * DP + kRC * kVS + kRC * kAS + DPAD * kVS + 66) * sizeof(float);
+}
+
 // grid (T, H): o[t][h][:] <- (unit ? o / rms(o) : o) * act(g[t * ldg + h * dv + :])
 __global__ void __launch_bounds__(256) head_gate_kernel(float* __restrict__ o, const float* __restrict__ g, long ldg,
                                                         int H, int dv, int unit, float eps, int act) {
@@ -255,7 +394,7 @@ __global__ void __launch_bounds__(256) latent_attention_kernel(LatAttArgs p) {
 
 extern "C" int lgs_retention(const float* q, const float* k, const float* v, long ld, float* state, const float* decay,
                              const float* inv_freq, const int* seq_start, const int* seq_slot, const int* seq_pos0,
-                             float* out, int B, int H, int d, int dv, int rot_dims, float k_scale,
+                             float* out, int B, int H, int d, int dv, int rot_dims, float k_scale, int chunked,
                              hipStream_t stream) {
   LGA_CHECK_ARG(q && k && v && state && decay && seq_start && seq_slot && seq_pos0 && out, "lgs_retention: null pointer");
   LGA_CHECK_ARG(B > 0 && H > 0 && H <= 65535 && d > 0 && d <= 256 && dv > 0, "lgs_retention: head dim must be in [1, 256]");
@@ -263,6 +402,20 @@ extern "C" int lgs_retention(const float* q, const float* k, const float* v, lon
                 "lgs_retention: bad rotary dims");
   lgs::RetArgs p{q, k, v, ld, state, decay, inv_freq, seq_start, seq_slot, seq_pos0, out, H, d, dv, rot_dims, k_scale};
   const dim3 grid(B, H, (dv + 63) / 64);
+  if (chunked && d <= 128) {  // a prompt: chunks of 64 tokens as fp32 matrix products
+    const size_t lds = lgs::retention_chunk_lds(d);
+    static size_t allowed = 0;
+    if (lds > allowed) {
+      if (hipFuncSetAttribute((const void*)lgs::retention_chunk_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)lds) != hipSuccess) {
+        lga_set_error("lgs_retention: cannot reserve the chunk kernel's LDS");
+        return (int)hipErrorInvalidValue;
+      }
+      allowed = lds;
+    }
+    lgs::retention_chunk_kernel<<<grid, 256, lds, stream>>>(p);
+    LGA_LAUNCH_RETURN();
+  }
   if (d <= 64) lgs::retention_scan_kernel<16><<<grid, 256, 0, stream>>>(p);
   else if (d <= 128) lgs::retention_scan_kernel<32><<<grid, 256, 0, stream>>>(p);
   else lgs::retention_scan_kernel<64><<<grid, 256, 0, stream>>>(p);
