@@ -65,10 +65,18 @@ int lgs_latent_prepare(float* proj, long ld, int q_off, int kv_off, void* cache_
                        int d, int dr, int r, int rot_dims, int max_seq, float eps, lgs_stream_t stream);
 /* out[t][h] = sum_j p_j c_j over cached rows j <= pos[t] of slot[t], p = softmax over
  * (qc[t][h] . c_j + q_rot[t][h] . kr_j) * scale with exp(sink[h]) added to the denominator (sink NULL: none).
- * r <= 512, dr <= 128. */
+ * r <= 512, dr <= 128. splits > 1 spreads every (token, head)'s keys over that many workgroups (decode: few rows,
+ * long contexts) and merges them in a second launch; part: T * H * splits * (r + 2) floats of workspace. */
 int lgs_latent_attention(const float* qc, const float* proj, long ld, int q_off, const void* cache_c, int cache_f32,
                          const float* cache_kr, const float* sink, const int* slot, const int* pos, float* out, int T,
-                         int H, int d, int dr, int r, int max_seq, float scale, lgs_stream_t stream);
+                         int H, int d, int dr, int r, int max_seq, float scale, int splits, float* part,
+                         lgs_stream_t stream);
+/* the prompt form of lgs_latent_attention: tiles of 16 consecutive tokens of one sequence and one head against key
+ * tiles of 16 cached rows, both products on fp32 MFMA; max_len = the most tokens any sequence brings. r % 64 == 0. */
+int lgs_latent_attention_tiles(const float* qc, const float* proj, long ld, int q_off, const void* cache_c,
+                               int cache_f32, const float* cache_kr, const float* sink, const int* seq_start,
+                               const int* seq_slot, const int* seq_pos0, float* out, int B, int max_len, int H, int d,
+                               int dr, int r, int max_seq, float scale, lgs_stream_t stream);
 
 /* out[t][i] = act(a[t * ld + i]) * b[t * ld + i], i < n */
 int lgs_glu(const float* a, const float* b, long ld, float* out, int T, int n, int act, lgs_stream_t stream);
@@ -80,9 +88,10 @@ int lgs_moe_up(const float* h, long ldh, const void* up, int w_f32, const int* i
                int F, int K, int act, lgs_stream_t stream);
 int lgs_moe_down(const float* actbuf, const void* down, int w_f32, const int* ids, const float* wts, float* x,
                  long ldx, int T, int top, int N, int F, lgs_stream_t stream);
-/* stable counting sort of the (token, choice) pairs by expert: z_start [E + 1], tok_of [pairs] (token of each sorted
- * entry), where [pairs] (sorted place of each pair) */
-int lgs_moe_sort(const int* ids, int pairs, int top, int E, int* z_start, int* tok_of, int* where,
+/* counting sort of the (token, choice) pairs by expert: z_start [E + 1], tok_of [pairs] (token of each sorted entry),
+ * where [pairs] (sorted place of each pair); the order inside an expert's range is not fixed. ws: 2 E ints, zero on
+ * entry, left zero. */
+int lgs_moe_sort(const int* ids, int pairs, int top, int E, int* z_start, int* tok_of, int* where, int* ws,
                  lgs_stream_t stream);
 /* x[t] += sum_k wts[t][k] * y[where[t * top + k]] */
 int lgs_moe_combine(const float* y, const int* where, const float* wts, float* x, long ldx, int T, int top, int N,

@@ -6,7 +6,7 @@
 //   lgs_moe_up / _down   the routed experts as streaming GEMVs over (token, choice) pairs: only the chosen experts'
 //                        rows are read; the down kernel sums a token's choices in their routing order and adds the
 //                        result to the residual stream (the decode form; a prompt runs grouped products instead)
-//   lgs_moe_sort / lgs_moe_combine   the prompt form: a stable counting sort of the (token, choice) pairs by
+//   lgs_moe_sort / lgs_moe_combine   the prompt form: a counting sort of the (token, choice) pairs by
 //                        expert, whose ranges drive lgs_linear's grouped products, and the weighted sum back
 //   lgs_token_side       per-layer token input: x += unit_rms(proj(gelu_tanh(gate x) * e[token])) * w
 #include "seq_common.h"
@@ -118,36 +118,58 @@ __global__ void __launch_bounds__(256) moe_down_kernel(const float* __restrict__
   }
 }
 
-// One workgroup: stable counting sort of the pairs by expert. z_start[E + 1] expert ranges in the sorted list,
-// tok_of[i] the token (row of h) of sorted entry i, where[pair] the sorted place of a pair.
-__global__ void __launch_bounds__(256) moe_sort_kernel(const int* __restrict__ ids, int pairs, int top, int E,
-                                                       int* __restrict__ z_start, int* __restrict__ tok_of,
-                                                       int* __restrict__ where) {
-  __shared__ int start[257];
+// Counting sort of the pairs by expert in three launches. ws: 2 E ints (counts, cursors), zero on entry.
+// z_start[E + 1] expert ranges in the sorted list, tok_of[i] the token (row of h) of sorted entry i, where[pair] the
+// sorted place of a pair. The order inside an expert's range is whatever the atomics give: every row of the grouped
+// products is computed on its own, so the sums do not depend on it.
+__global__ void __launch_bounds__(256) moe_count_kernel(const int* __restrict__ ids, int pairs, int E, int* __restrict__ ws) {
+  __shared__ int lh[256];
+  lh[threadIdx.x] = 0;
+  __syncthreads();
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < pairs) atomicAdd(&lh[ids[i]], 1);
+  __syncthreads();
+  if (threadIdx.x < E && lh[threadIdx.x]) atomicAdd(&ws[threadIdx.x], lh[threadIdx.x]);
+}
+
+__global__ void __launch_bounds__(256) moe_scan_kernel(int E, int* __restrict__ ws, int* __restrict__ z_start) {
+  __shared__ int cnt[256];
   const int tid = threadIdx.x;
-  // thread e counts expert e (E <= 256): a plain pass keeps the order stable and needs no atomics
-  int cnt = 0;
-  if (tid < E)
-    for (int i = 0; i < pairs; ++i) cnt += ids[i] == tid;
-  if (tid == 0) start[0] = 0;
+  cnt[tid] = tid < E ? ws[tid] : 0;
   __syncthreads();
-  // prefix over at most 256 counts by one thread per step would be slow; E is small, thread 0 scans
-  __shared__ int counts[256];
-  counts[tid] = tid < E ? cnt : 0;
-  __syncthreads();
-  if (tid == 0)
-    for (int e = 0; e < E; ++e) start[e + 1] = start[e] + counts[e];
-  __syncthreads();
-  if (tid < E) z_start[tid] = start[tid];
-  if (tid == 0) z_start[E] = start[E];
+  if (tid == 0) {
+    int at = 0;
+    for (int e = 0; e < E; ++e) {
+      z_start[e] = at;
+      at += cnt[e];
+    }
+    z_start[E] = at;
+  }
   if (tid < E) {
-    int at = start[tid];
-    for (int i = 0; i < pairs; ++i)
-      if (ids[i] == tid) {
-        tok_of[at] = i / top;
-        where[i] = at;
-        ++at;
-      }
+    ws[tid] = 0;      // counts: zero again for the next call
+    ws[E + tid] = 0;  // cursors
+  }
+}
+
+__global__ void __launch_bounds__(256) moe_place_kernel(const int* __restrict__ ids, int pairs, int top, int E,
+                                                        const int* __restrict__ z_start, int* __restrict__ ws,
+                                                        int* __restrict__ tok_of, int* __restrict__ where) {
+  __shared__ int lh[256], base[256];
+  lh[threadIdx.x] = 0;
+  __syncthreads();
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  int e = 0, rank = 0;
+  if (i < pairs) {
+    e = ids[i];
+    rank = atomicAdd(&lh[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x < E && lh[threadIdx.x]) base[threadIdx.x] = atomicAdd(&ws[E + threadIdx.x], lh[threadIdx.x]);
+  __syncthreads();
+  if (i < pairs) {
+    const int at = z_start[e] + base[e] + rank;
+    tok_of[at] = i / top;
+    where[i] = at;
   }
 }
 
@@ -236,11 +258,14 @@ extern "C" int lgs_moe_down(const float* actbuf, const void* down, int w_f32, co
   LGA_LAUNCH_RETURN();
 }
 
-extern "C" int lgs_moe_sort(const int* ids, int pairs, int top, int E, int* z_start, int* tok_of, int* where,
+extern "C" int lgs_moe_sort(const int* ids, int pairs, int top, int E, int* z_start, int* tok_of, int* where, int* ws,
                             hipStream_t stream) {
-  LGA_CHECK_ARG(ids && z_start && tok_of && where && pairs > 0 && top > 0 && E > 0 && E <= 256,
+  LGA_CHECK_ARG(ids && z_start && tok_of && where && ws && pairs > 0 && top > 0 && E > 0 && E <= 256,
                 "lgs_moe_sort: experts must be <= 256");
-  lgs::moe_sort_kernel<<<1, 256, 0, stream>>>(ids, pairs, top, E, z_start, tok_of, where);
+  const int blocks = (pairs + 255) / 256;
+  lgs::moe_count_kernel<<<blocks, 256, 0, stream>>>(ids, pairs, E, ws);
+  lgs::moe_scan_kernel<<<1, 256, 0, stream>>>(E, ws, z_start);
+  lgs::moe_place_kernel<<<blocks, 256, 0, stream>>>(ids, pairs, top, E, z_start, ws, tok_of, where);
   LGA_LAUNCH_RETURN();
 }
 

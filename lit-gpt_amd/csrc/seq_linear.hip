@@ -29,9 +29,9 @@ struct LinArgs {
 };
 
 // ------------------------------------------------------------------------------------------------ GEMV, M <= 8
-template <bool WF32, int MT>
+// R output columns per wave: 4 for tall matrices (more loads in flight per lane), fewer for short ones (more waves)
+template <bool WF32, int MT, int R>
 __global__ void __launch_bounds__(256) lin_gemv_kernel(LinArgs p) {
-  constexpr int R = 2;  // output columns per wave
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int z = blockIdx.y;
   const int n0 = (blockIdx.x * 4 + wave) * R;
@@ -50,6 +50,7 @@ __global__ void __launch_bounds__(256) lin_gemv_kernel(LinArgs p) {
 #pragma unroll
   for (int r = 0; r < R; ++r) rows[r] = min(n0 + r, p.N - 1);
   if (vec) {
+#pragma unroll 2
     for (int k = lane * 8; k < K; k += 512) {
       float wv[R][8];
 #pragma unroll
@@ -334,17 +335,25 @@ extern "C" int lgs_linear(const float* a, long lda, long stride_a, const void* w
   LGA_CHECK_ARG(act >= 0 && act <= lgs::kActSigmoid, "lgs_linear: unknown activation");
   lgs::LinArgs p{a, lda, stride_a, w, stride_w, y, ldy, stride_y, M, N, K, accumulate, act, a_rows, z_start};
   if (M <= 8 && !z_start && !a_rows) {
-    const dim3 grid((N + 7) / 8, batch);
-#define LGS_GEMV(MT)                                                                  \
-  do {                                                                                \
-    if (w_f32) lgs::lin_gemv_kernel<true, MT><<<grid, 256, 0, stream>>>(p);           \
-    else lgs::lin_gemv_kernel<false, MT><<<grid, 256, 0, stream>>>(p);                \
+    const int R = N >= 16384 ? 4 : (N >= 4096 ? 2 : 1);
+    const dim3 grid((N + 4 * R - 1) / (4 * R), batch);
+#define LGS_GEMV_R(MT, RR)                                                              \
+  do {                                                                                  \
+    if (w_f32) lgs::lin_gemv_kernel<true, MT, RR><<<grid, 256, 0, stream>>>(p);         \
+    else lgs::lin_gemv_kernel<false, MT, RR><<<grid, 256, 0, stream>>>(p);              \
+  } while (0)
+#define LGS_GEMV(MT)                 \
+  do {                               \
+    if (R == 4) LGS_GEMV_R(MT, 4);   \
+    else if (R == 2) LGS_GEMV_R(MT, 2); \
+    else LGS_GEMV_R(MT, 1);          \
   } while (0)
     if (M == 1) LGS_GEMV(1);
     else if (M == 2) LGS_GEMV(2);
     else if (M <= 4) LGS_GEMV(4);
     else LGS_GEMV(8);
 #undef LGS_GEMV
+#undef LGS_GEMV_R
     LGA_LAUNCH_RETURN();
   }
   if (w_f32) {

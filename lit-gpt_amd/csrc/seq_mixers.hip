@@ -324,15 +324,21 @@ struct LatAttArgs {
   float scale;
 };
 
-// grid (T, H): wave w walks keys w, w + 4, ... <= pos with an online softmax; lanes hold dims lane + 64 e
+// grid (T, H, splits): split z of (token, head) owns an equal share of the keys 0 .. pos; its wave w walks keys
+// lo + w, lo + w + 4, ... four at a time (their loads in flight together) with an online softmax; lanes hold dims
+// lane + 64 e. One split finishes in place (the sink joins the denominator); several leave (max, sum, weighted sum)
+// per split in `part` [T][H][splits][r + 2] for latent_combine_kernel.
 template <bool CF32, int NR>
-__global__ void __launch_bounds__(256) latent_attention_kernel(LatAttArgs p) {
+__global__ void __launch_bounds__(256) latent_attention_kernel(LatAttArgs p, float* __restrict__ part) {
   __shared__ float sm[4], sl[4];
   extern __shared__ float sacc[];  // [4][r]
-  const int t = blockIdx.x, h = blockIdx.y;
+  constexpr int U = 4;
+  const int t = blockIdx.x, h = blockIdx.y, z = blockIdx.z, splits = gridDim.z;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r = p.r, dr = p.dr;
   const int last = min(p.pos[t], p.max_seq - 1);
+  const int share = (last + splits) / splits;  // ceil((last + 1) / splits)
+  const int lo = z * share, hi = min(last, lo + share - 1);
   const size_t base = (size_t)p.slot[t] * p.max_seq;
   const float* qc = p.qc + ((size_t)t * p.H + h) * r;
   const float* qr = p.proj + (size_t)t * p.ld + p.q_off + (size_t)h * (p.d + dr) + p.d;
@@ -345,29 +351,41 @@ __global__ void __launch_bounds__(256) latent_attention_kernel(LatAttArgs p) {
 #pragma unroll
   for (int e = 0; e < 2; ++e) qrot[e] = lane + 64 * e < dr ? qr[lane + 64 * e] : 0.0f;
   float m = -INFINITY, l = 0.0f;
-  for (int j = wave; j <= last; j += 4) {
-    float c[NR];
-    float dot = 0.0f;
+  for (int j0 = lo + wave; j0 <= hi; j0 += 4 * U) {
+    float c[U][NR], dot[U];
 #pragma unroll
-    for (int e = 0; e < NR; ++e) {
-      const int i = lane + 64 * e;
-      c[e] = i < r ? (CF32 ? ((const float*)p.cache_c)[(base + j) * r + i]
-                           : bf2f(((const uint16_t*)p.cache_c)[(base + j) * r + i]))
-                   : 0.0f;
-      dot = fmaf(q[e], c[e], dot);
+    for (int u = 0; u < U; ++u) {
+      const int j = min(j0 + 4 * u, hi);  // a key past the end repeats the last one and gets no weight
+      dot[u] = 0.0f;
+#pragma unroll
+      for (int e = 0; e < NR; ++e) {
+        const int i = lane + 64 * e;
+        c[u][e] = i < r ? (CF32 ? ((const float*)p.cache_c)[(base + j) * r + i]
+                                : bf2f(((const uint16_t*)p.cache_c)[(base + j) * r + i]))
+                        : 0.0f;
+      }
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const int i = lane + 64 * e;
+        if (i < dr) dot[u] = fmaf(qrot[e], p.cache_kr[(base + j) * dr + i], dot[u]);
+      }
     }
 #pragma unroll
-    for (int e = 0; e < 2; ++e) {
-      const int i = lane + 64 * e;
-      if (i < dr) dot = fmaf(qrot[e], p.cache_kr[(base + j) * dr + i], dot);
-    }
-    const float s = wave_sum(dot) * p.scale;
-    const float mn = fmaxf(m, s);
-    const float corr = expf(m - mn), w = expf(s - mn);
-    l = l * corr + w;
+    for (int u = 0; u < U; ++u) {
 #pragma unroll
-    for (int e = 0; e < NR; ++e) acc[e] = acc[e] * corr + w * c[e];
-    m = mn;
+      for (int e = 0; e < NR; ++e) dot[u] = fmaf(q[e], c[u][e], dot[u]);
+      dot[u] = wave_sum(dot[u]) * p.scale;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (j0 + 4 * u > hi) break;
+      const float mn = fmaxf(m, dot[u]);
+      const float corr = expf(m - mn), w = expf(dot[u] - mn);
+      l = l * corr + w;
+#pragma unroll
+      for (int e = 0; e < NR; ++e) acc[e] = acc[e] * corr + w * c[u][e];
+      m = mn;
+    }
   }
   if (lane == 0) {
     sm[wave] = m;
@@ -377,17 +395,216 @@ __global__ void __launch_bounds__(256) latent_attention_kernel(LatAttArgs p) {
   for (int e = 0; e < NR; ++e)
     if (lane + 64 * e < r) sacc[wave * r + lane + 64 * e] = acc[e];
   __syncthreads();
-  const float snk = p.sink ? p.sink[h] : -INFINITY;
+  const bool fin = splits == 1;
+  const float snk = (fin && p.sink) ? p.sink[h] : -INFINITY;
   const float mx = fmaxf(fmaxf(fmaxf(sm[0], sm[1]), fmaxf(sm[2], sm[3])), snk);
-  float f[4], den = p.sink ? expf(snk - mx) : 0.0f;
+  float f[4], den = (fin && p.sink) ? expf(snk - mx) : 0.0f;
 #pragma unroll
   for (int w = 0; w < 4; ++w) {
     f[w] = sl[w] > 0.0f ? expf(sm[w] - mx) : 0.0f;
     den += sl[w] * f[w];
   }
-  float* o = p.out + ((size_t)t * p.H + h) * r;
-  for (int i = threadIdx.x; i < r; i += 256)
-    o[i] = ((sacc[i] * f[0] + sacc[r + i] * f[1]) + (sacc[2 * r + i] * f[2] + sacc[3 * r + i] * f[3])) / den;
+  if (fin) {
+    float* o = p.out + ((size_t)t * p.H + h) * r;
+    for (int i = threadIdx.x; i < r; i += 256)
+      o[i] = ((sacc[i] * f[0] + sacc[r + i] * f[1]) + (sacc[2 * r + i] * f[2] + sacc[3 * r + i] * f[3])) / den;
+  } else {
+    float* o = part + (((size_t)t * p.H + h) * splits + z) * (r + 2);
+    if (threadIdx.x == 0) {
+      o[0] = mx;
+      o[1] = den;
+    }
+    for (int i = threadIdx.x; i < r; i += 256)
+      o[2 + i] = (sacc[i] * f[0] + sacc[r + i] * f[1]) + (sacc[2 * r + i] * f[2] + sacc[3 * r + i] * f[3]);
+  }
+}
+
+// The prompt form: 16 consecutive tokens of one sequence and one head per workgroup, key tiles of 16 cached rows
+// staged in LDS as fp32, both products on v_mfma_f32_16x16x4_f32. The four waves split the score product over the
+// latent / rotated dims (partial 16x16 tiles summed through LDS) and the weighted sum over the r output columns
+// (NT tiles of 16 per wave); each runs the same online softmax on the summed scores. The next key tile travels in
+// registers while the current one is multiplied. r % 64 == 0.
+struct LatTileArgs {
+  LatAttArgs a;
+  const int* seq_start;
+  const int* seq_slot;
+  const int* seq_pos0;
+};
+
+template <bool CF32, int NT>
+__global__ void __launch_bounds__(256) latent_attention_tile_kernel(LatTileArgs tp) {
+  extern __shared__ float lds[];
+  const LatAttArgs& p = tp.a;
+  const int b = blockIdx.z, h = blockIdx.y;
+  const int t0 = tp.seq_start[b] + blockIdx.x * 16, t1 = tp.seq_start[b + 1];
+  if (t0 >= t1) return;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, fr = lane & 15, fk = lane >> 4;
+  const int r = p.r, dr = p.dr, D = r + dr;
+  const int DQ = (D + 15) / 16 * 4;             // dims per wave in the score product (multiple of 4)
+  const int KP = (4 * DQ + 31) / 32 * 32 + 2;   // row stride of the Q and key tiles (conflict-free 16 x 4 reads)
+  float* Qt = lds;                  // [16][KP]
+  float* Kt = Qt + 16 * KP;         // [16][KP]
+  float* Sp = Kt + 16 * KP;         // [4][16][17] partial scores
+  float* Pw = Sp + 4 * 16 * 17;     // [4][16][17] each wave's copy of the weights
+  const int rows = min(16, t1 - t0);
+  const int pos_first = tp.seq_pos0[b] + blockIdx.x * 16;
+  const int pos_last = min(pos_first + rows - 1, p.max_seq - 1);
+  const size_t base = (size_t)tp.seq_slot[b] * p.max_seq;
+  for (int i = tid; i < 16 * KP; i += 256) {
+    const int row = i / KP, dd = i - row * KP;
+    float v = 0.0f;
+    if (row < rows) {
+      if (dd < r) v = p.qc[((size_t)(t0 + row) * p.H + h) * r + dd];
+      else if (dd < D) v = p.proj[(size_t)(t0 + row) * p.ld + p.q_off + (size_t)h * (p.d + dr) + p.d + (dd - r)];
+    }
+    Qt[i] = v;
+    Kt[i] = 0.0f;  // the padding columns stay zero; the live ones are rewritten per tile
+  }
+  constexpr int NC = CF32 ? 8 : 4;  // 16-B loads of the latent part per thread (r <= 512)
+  uint4 creg[NC];
+  float kreg[8];
+  const int cvec = CF32 ? r / 4 : r / 8;  // 16-B vectors per cached latent row
+  auto gload = [&](int kt) {
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+      const int idx = tid + 256 * i;
+      if (idx < 16 * cvec) {
+        const int key = min(kt * 16 + idx / cvec, p.max_seq - 1), v = idx % cvec;
+        creg[i] = CF32 ? ((const uint4*)((const float*)p.cache_c + (base + key) * r))[v]
+                       : ((const uint4*)((const uint16_t*)p.cache_c + (base + key) * r))[v];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int idx = tid + 256 * i;
+      if (idx < 16 * dr) kreg[i] = p.cache_kr[(base + min(kt * 16 + idx / dr, p.max_seq - 1)) * dr + idx % dr];
+    }
+  };
+  auto lstore = [&]() {
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+      const int idx = tid + 256 * i;
+      if (idx < 16 * cvec) {
+        const int key = idx / cvec, v = idx % cvec;
+        float* dst = Kt + key * KP + v * (CF32 ? 4 : 8);
+        const uint32_t w[4] = {creg[i].x, creg[i].y, creg[i].z, creg[i].w};
+        if (CF32) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) dst[e] = __uint_as_float(w[e]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            dst[2 * e] = bflo(w[e]);
+            dst[2 * e + 1] = bfhi(w[e]);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int idx = tid + 256 * i;
+      if (idx < 16 * dr) Kt[(idx / dr) * KP + r + idx % dr] = kreg[i];
+    }
+  };
+  f32x4_t o[NT];
+#pragma unroll
+  for (int c = 0; c < NT; ++c) o[c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  float m[4], l[4];
+  int prow[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    m[j] = -INFINITY;
+    l[j] = 0.0f;
+    prow[j] = min(pos_first + fk * 4 + j, pos_last);  // rows past the sequence's end repeat the last (not stored)
+  }
+  const int nkt = pos_last / 16 + 1;
+  gload(0);
+  __syncthreads();  // Qt, and Kt's zero padding
+  for (int kt = 0; kt < nkt; ++kt) {
+    lstore();
+    __syncthreads();
+    if (kt + 1 < nkt) gload(kt + 1);
+    // partial scores over this wave's dims
+    f32x4_t sacc = {0.f, 0.f, 0.f, 0.f};
+    const float* qa = Qt + fr * KP + wave * DQ + fk;
+    const float* kb = Kt + fr * KP + wave * DQ + fk;
+    for (int k = 0; k < DQ; k += 4) sacc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[k], kb[k], sacc, 0, 0, 0);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) Sp[(wave * 16 + fk * 4 + j) * 17 + fr] = sacc[j];
+    __syncthreads();
+    float pj[4], corr[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int row = fk * 4 + j;
+      float sc = ((Sp[row * 17 + fr] + Sp[(16 + row) * 17 + fr]) + (Sp[(32 + row) * 17 + fr] + Sp[(48 + row) * 17 + fr])) *
+                 p.scale;
+      if (kt * 16 + fr > prow[j]) sc = -INFINITY;
+      float mx = sc;
+#pragma unroll
+      for (int x = 8; x > 0; x >>= 1) mx = fmaxf(mx, __shfl_xor(mx, x));
+      const float mn = fmaxf(m[j], mx);
+      const float w = expf(sc - mn);
+      float sum = w;
+#pragma unroll
+      for (int x = 8; x > 0; x >>= 1) sum += __shfl_xor(sum, x);
+      corr[j] = expf(m[j] - mn);
+      l[j] = l[j] * corr[j] + sum;
+      m[j] = mn;
+      pj[j] = w;
+      Pw[(wave * 16 + row) * 17 + fr] = w;
+    }
+#pragma unroll
+    for (int c = 0; c < NT; ++c)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[c][j] *= corr[j];
+    __syncthreads();
+    // weighted sum of the cached latents: this wave's NT column tiles
+    const float* pa = Pw + (wave * 16 + fr) * 17 + fk;
+#pragma unroll
+    for (int k = 0; k < 16; k += 4) {
+      const float a = pa[k];
+      const float* vb = Kt + (k + fk) * KP + wave * NT * 16 + fr;
+#pragma unroll
+      for (int c = 0; c < NT; ++c) o[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, vb[c * 16], o[c], 0, 0, 0);
+    }
+    __syncthreads();  // Kt and Sp are free for the next tile
+  }
+  const float snk = p.sink ? p.sink[h] : -INFINITY;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int row = fk * 4 + j;
+    if (row >= rows) continue;
+    const float mx = fmaxf(m[j], snk);
+    const float f = expf(m[j] - mx);
+    const float den = l[j] * f + (p.sink ? expf(snk - mx) : 0.0f);
+    float* orow = p.out + ((size_t)(t0 + row) * p.H + h) * r + wave * NT * 16 + fr;
+#pragma unroll
+    for (int c = 0; c < NT; ++c) orow[c * 16] = o[c][j] * f / den;
+  }
+}
+
+// grid (T, H): merges the splits' partial softmaxes and the sink
+__global__ void __launch_bounds__(256) latent_combine_kernel(const float* __restrict__ part, const float* __restrict__ sink,
+                                                             float* __restrict__ out, int H, int r, int splits) {
+  const int t = blockIdx.x, h = blockIdx.y;
+  const float* pp = part + ((size_t)t * H + h) * splits * (r + 2);
+  const float snk = sink ? sink[h] : -INFINITY;
+  float mx = snk;
+  for (int z = 0; z < splits; ++z)
+    if (pp[(size_t)z * (r + 2) + 1] > 0.0f) mx = fmaxf(mx, pp[(size_t)z * (r + 2)]);
+  float den = sink ? expf(snk - mx) : 0.0f;
+  for (int z = 0; z < splits; ++z) {
+    const float lz = pp[(size_t)z * (r + 2) + 1];
+    if (lz > 0.0f) den += lz * expf(pp[(size_t)z * (r + 2)] - mx);
+  }
+  for (int i = threadIdx.x; i < r; i += 256) {
+    float a = 0.0f;
+    for (int z = 0; z < splits; ++z) {
+      const float lz = pp[(size_t)z * (r + 2) + 1];
+      if (lz > 0.0f) a += pp[(size_t)z * (r + 2) + 2 + i] * expf(pp[(size_t)z * (r + 2)] - mx);
+    }
+    out[((size_t)t * H + h) * r + i] = a / den;
+  }
 }
 
 }  // namespace lgs
@@ -447,21 +664,64 @@ extern "C" int lgs_latent_prepare(float* proj, long ld, int q_off, int kv_off, v
 extern "C" int lgs_latent_attention(const float* qc, const float* proj, long ld, int q_off, const void* cache_c,
                                     int cache_f32, const float* cache_kr, const float* sink, const int* slot,
                                     const int* pos, float* out, int T, int H, int d, int dr, int r, int max_seq,
-                                    float scale, hipStream_t stream) {
+                                    float scale, int splits, float* part, hipStream_t stream) {
   LGA_CHECK_ARG(qc && proj && cache_c && cache_kr && slot && pos && out, "lgs_latent_attention: null pointer");
   LGA_CHECK_ARG(T > 0 && H > 0 && H <= 65535 && r > 0 && r <= 512 && dr >= 0 && dr <= 128 && max_seq > 0,
                 "lgs_latent_attention: latent rank must be <= 512 and the rotated part <= 128");
+  LGA_CHECK_ARG(splits >= 1 && splits <= 256 && (splits == 1 || part),
+                "lgs_latent_attention: splits in [1, 256], with a workspace of T * H * splits * (r + 2) floats");
   lgs::LatAttArgs p{qc, proj, ld, q_off, cache_c, cache_kr, sink, slot, pos, out, H, d, dr, r, max_seq, scale};
-  const dim3 grid(T, H);
+  const dim3 grid(T, H, splits);
   const size_t lds = (size_t)4 * r * sizeof(float);
-#define LGS_LAT(NR)                                                                              \
-  do {                                                                                           \
-    if (cache_f32) lgs::latent_attention_kernel<true, NR><<<grid, 256, lds, stream>>>(p);        \
-    else lgs::latent_attention_kernel<false, NR><<<grid, 256, lds, stream>>>(p);                 \
+#define LGS_LAT(NR)                                                                                    \
+  do {                                                                                                 \
+    if (cache_f32) lgs::latent_attention_kernel<true, NR><<<grid, 256, lds, stream>>>(p, part);        \
+    else lgs::latent_attention_kernel<false, NR><<<grid, 256, lds, stream>>>(p, part);                 \
   } while (0)
   if (r <= 128) LGS_LAT(2);
   else if (r <= 256) LGS_LAT(4);
   else LGS_LAT(8);
 #undef LGS_LAT
+  if (splits > 1) lgs::latent_combine_kernel<<<dim3(T, H), 256, 0, stream>>>(part, sink, out, H, r, splits);
+  LGA_LAUNCH_RETURN();
+}
+
+extern "C" int lgs_latent_attention_tiles(const float* qc, const float* proj, long ld, int q_off, const void* cache_c,
+                                          int cache_f32, const float* cache_kr, const float* sink,
+                                          const int* seq_start, const int* seq_slot, const int* seq_pos0, float* out,
+                                          int B, int max_len, int H, int d, int dr, int r, int max_seq, float scale,
+                                          hipStream_t stream) {
+  LGA_CHECK_ARG(qc && proj && cache_c && cache_kr && seq_start && seq_slot && seq_pos0 && out,
+                "lgs_latent_attention_tiles: null pointer");
+  LGA_CHECK_ARG(B > 0 && B <= 65535 && max_len > 0 && H > 0 && H <= 65535 && max_seq > 0,
+                "lgs_latent_attention_tiles: bad sizes");
+  LGA_CHECK_ARG(r > 0 && r <= 512 && r % 64 == 0 && dr >= 0 && dr <= 128,
+                "lgs_latent_attention_tiles: latent rank must be a multiple of 64 up to 512, the rotated part <= 128");
+  lgs::LatTileArgs p{{qc, proj, ld, q_off, cache_c, cache_kr, sink, nullptr, nullptr, out, H, d, dr, r, max_seq, scale},
+                     seq_start, seq_slot, seq_pos0};
+  const int D = r + dr, DQ = (D + 15) / 16 * 4, KP = (4 * DQ + 31) / 32 * 32 + 2;
+  const size_t lds = (size_t)(2 * 16 * KP + 2 * 4 * 16 * 17) * sizeof(float);
+  const dim3 grid((max_len + 15) / 16, H, B);
+  const void* fn = nullptr;
+#define LGS_TILE(NT)                                                                                   \
+  case NT:                                                                                             \
+    fn = cache_f32 ? (const void*)lgs::latent_attention_tile_kernel<true, NT>                          \
+                   : (const void*)lgs::latent_attention_tile_kernel<false, NT>;                        \
+    break;
+  switch (r / 64) {
+    LGS_TILE(1) LGS_TILE(2) LGS_TILE(3) LGS_TILE(4) LGS_TILE(5) LGS_TILE(6) LGS_TILE(7) LGS_TILE(8)
+  }
+#undef LGS_TILE
+  if (lds > 48 * 1024 &&
+      hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
+    lga_set_error("lgs_latent_attention_tiles: cannot reserve the kernel's LDS");
+    return (int)hipErrorInvalidValue;
+  }
+  void* args[] = {(void*)&p};
+  hipError_t e = hipLaunchKernel(fn, grid, dim3(256), args, lds, stream);
+  if (e != hipSuccess) {
+    lga_set_error(hipGetErrorString(e));
+    return (int)e;
+  }
   LGA_LAUNCH_RETURN();
 }

@@ -83,12 +83,26 @@ class BatchEngine:
             self.pool.give(slot)
         return out
 
+    def decode_graph(self, requests: Sequence[Hashable], tokens: Sequence[int]) -> "GreedyDecodeGraph":
+        """A captured greedy decode step for these live requests, whose next input tokens are ``tokens``."""
+        return GreedyDecodeGraph(self, requests, tokens)
+
     @torch.inference_mode()
     def generate(self, prompts: Sequence[Sequence[int]], max_new_tokens: int, *, temperature: float = 0.0,
-                 top_k: Optional[int] = None, eos_id: Optional[int] = None) -> List[List[int]]:
+                 top_k: Optional[int] = None, eos_id: Optional[int] = None, use_graph: bool = False) -> List[List[int]]:
         """Continue every prompt by up to ``max_new_tokens`` tokens: one prompt step for all, then one-token steps
-        for those still running (a request that drew ``eos_id`` leaves the batch). Returns prompt + continuation."""
+        for those still running (a request that drew ``eos_id`` leaves the batch). Returns prompt + continuation.
+        ``use_graph`` (greedy, no eos): the one-token steps run as replays of one captured HIP graph."""
         from generate.base import sample
+
+        if use_graph and temperature == 0.0 and eos_id is None and max_new_tokens > 1:
+            ids = [object() for _ in prompts]
+            logits = self.step([(ids[i], list(p), [len(p) - 1]) for i, p in enumerate(prompts)])
+            first = [int(sample(logits[i].view(1, 1, -1), temperature=0.0)) for i in range(len(prompts))]
+            graph = self.decode_graph(ids, first)
+            new = torch.stack([graph.step().clone() for _ in range(max_new_tokens - 1)]).cpu()
+            self.step([], end=ids)
+            return [list(p) + [first[i]] + new[:, i].tolist() for i, p in enumerate(prompts)]
 
         ids = [object() for _ in prompts]
         seqs = [list(p) for p in prompts]
@@ -112,3 +126,56 @@ class BatchEngine:
             if not running:
                 break
         return seqs
+
+
+class GreedyDecodeGraph:
+    """One-token greedy steps of a fixed set of live requests as replays of one HIP graph: the step's table (tokens,
+    slots, positions) lives in static device buffers; the captured chain runs the model's step function, the output
+    product, the framework's argmax per row (which writes the next input token in place) and advances the positions
+    on the device, so a replay needs no host work. ``step()`` returns the (B,) device tensor of the tokens drawn."""
+
+    def __init__(self, engine: BatchEngine, requests: Sequence[Hashable], tokens: Sequence[int]) -> None:
+        from lit_gpt import ops
+
+        model, dev = engine.model, engine.device
+        self.engine, self.requests = engine, list(requests)
+        B = len(self.requests)
+        table = [(engine.live[r][0], engine.live[r][1], [int(t)]) for r, t in zip(self.requests, tokens)]
+        self.batch = StepBatch.build(table, dev)
+        self.drawn = torch.zeros(B, dtype=torch.int64, device=dev)
+        self.steps_done = 0
+        self.room = min(model.max_seq_length - engine.live[r][1] for r in self.requests)
+
+        def body() -> None:
+            b = self.batch
+            logits = model.logits(model.forward_step(b))
+            for i in range(B):
+                ops.argmax(logits[i], out_idx=self.drawn[i:i + 1], token_out=b.tokens[i:i + 1])
+            b.pos.add_(1)
+            b.seq_pos0.add_(1)
+
+        with torch.inference_mode():
+            body()  # the first step runs eagerly (it also builds every kernel's device object)
+            self._advance()
+            self.first = self.drawn.clone()
+            torch.cuda.synchronize(dev)
+            self.graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(self.graph):
+                body()
+        self._pending_first = True
+
+    def _advance(self) -> None:
+        if self.steps_done >= self.room:
+            raise ValueError("a request would outgrow the cache")
+        self.steps_done += 1
+        for r in self.requests:
+            slot, held = self.engine.live[r]
+            self.engine.live[r] = (slot, held + 1)
+
+    def step(self) -> torch.Tensor:
+        if self._pending_first:  # the eager step's tokens
+            self._pending_first = False
+            return self.first
+        self._advance()
+        self.graph.replay()
+        return self.drawn

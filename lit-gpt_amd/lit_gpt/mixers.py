@@ -34,6 +34,7 @@ class StepBatch:
     seq_pos0: torch.Tensor  # (B,) position of each sequence's first row
     T: int
     B: int
+    max_len: int = 0  # the most tokens any sequence brings to this step (host side; 0: unknown, taken as T)
 
     @classmethod
     def build(cls, entries: Sequence[Tuple[int, int, Sequence[int]]], device: torch.device) -> "StepBatch":
@@ -53,7 +54,7 @@ class StepBatch:
         flat = torch.tensor(tokens + slot + pos + start + sslot + spos, dtype=torch.int32).to(device)
         cut = [T, T, T, B + 1, B, B]
         parts = torch.split(flat, cut)
-        return cls(*parts, T=T, B=B)
+        return cls(*parts, T=T, B=B, max_len=max(len(e[2]) for e in entries))
 
 
 def _f32(t: torch.Tensor, device) -> torch.Tensor:
@@ -147,8 +148,13 @@ class LatentAttention(InputReader):
         qc = torch.empty(T, H * r, dtype=torch.float32, device=proj.device)
         seq_ops.linear(proj, self.w_ukT, M=T, N=r, K=d, y=qc, a_off=q_off, lda=ld, ldy=H * r, batch=H,
                        stride_a=d + dr, stride_w=r * d, stride_y=r)
-        lat = seq_ops.latent_attention(qc, proj, q_off, cache.c, cache.kr, self.sink, step.slot, step.pos, H=H, d=d,
-                                       dr=dr, r=r, scale=self.scale)
+        if r % 64 == 0 and T >= 8 * step.B:  # a prompt: 16-token tiles on the matrix cores
+            lat = seq_ops.latent_attention_tiles(qc, proj, q_off, cache.c, cache.kr, self.sink, step.seq_start,
+                                                 step.seq_slot, step.seq_pos0, step.max_len or T, H=H, d=d, dr=dr,
+                                                 r=r, scale=self.scale)
+        else:
+            lat = seq_ops.latent_attention(qc, proj, q_off, cache.c, cache.kr, self.sink, step.slot, step.pos, H=H,
+                                           d=d, dr=dr, r=r, scale=self.scale)
         att = torch.empty(T, H * dv, dtype=torch.float32, device=proj.device)
         seq_ops.linear(lat, self.w_uv, M=T, N=dv, K=r, y=att, lda=H * r, ldy=H * dv, batch=H, stride_a=r,
                        stride_w=dv * r, stride_y=dv)

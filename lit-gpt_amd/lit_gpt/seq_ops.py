@@ -38,12 +38,13 @@ SIGNATURES = {
     "lgs_retention": [_P, _P, _P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P],
     "lgs_head_gate": [_P, _P, _L, _I, _I, _I, _I, _F, _I, _P],
     "lgs_latent_prepare": [_P, _L, _I, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P],
-    "lgs_latent_attention": [_P, _P, _L, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P],
+    "lgs_latent_attention": [_P, _P, _L, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P],
+    "lgs_latent_attention_tiles": [_P, _P, _L, _I, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P],
     "lgs_glu": [_P, _P, _L, _P, _I, _I, _I, _P],
     "lgs_moe_route": [_P, _L, _I, _I, _I, _P, _P, _P],
     "lgs_moe_up": [_P, _L, _P, _I, _P, _P, _I, _I, _I, _I, _I, _P],
     "lgs_moe_down": [_P, _P, _I, _P, _P, _P, _L, _I, _I, _I, _I, _P],
-    "lgs_moe_sort": [_P, _I, _I, _I, _P, _P, _P, _P],
+    "lgs_moe_sort": [_P, _I, _I, _I, _P, _P, _P, _P, _P],
     "lgs_moe_combine": [_P, _P, _P, _P, _L, _I, _I, _I, _P],
     "lgs_token_side": [_P, _P, _P, _I, _L, _I, _P, _P, _P, _I, _I, _I, _I, _F, _P],
 }
@@ -193,17 +194,43 @@ def latent_prepare(proj: torch.Tensor, q_off: int, kv_off: int, cache_c: torch.T
 
 def latent_attention(qc: torch.Tensor, proj: torch.Tensor, q_off: int, cache_c: torch.Tensor, cache_kr: torch.Tensor,
                      sink: Optional[torch.Tensor], slot: torch.Tensor, pos: torch.Tensor, *, H: int, d: int, dr: int,
-                     r: int, scale: float) -> torch.Tensor:
+                     r: int, scale: float, splits: Optional[int] = None) -> torch.Tensor:
+    """Softmax attention of every (token, head) over its sequence's cached rows up to the token's position, in the
+    latent space. ``splits``: workgroups per (token, head); by default enough of them to fill the chip when the
+    step has few rows (decode), one when it has many (a prompt)."""
     T, ld = proj.shape
     S = cache_c.shape[1]
     if qc.shape != (T, H * r) or (sink is not None and sink.numel() != H):
         raise ValueError("latent_attention: shapes")
     out = torch.empty(T, H * r, dtype=F32, device=proj.device)
+    if splits is None:
+        splits = max(1, min(32, 1024 // (T * H)))
+    part = torch.empty(T * H * splits * (r + 2), dtype=F32, device=proj.device) if splits > 1 else None
     _check(load_library().lgs_latent_attention(_dev(qc, "qc", F32), _dev(proj, "proj", F32), ld, q_off,
                                                _dev(cache_c, "cache_c"), _wf32(cache_c, "cache_c"),
                                                _dev(cache_kr, "cache_kr", F32), _opt(sink, "sink", F32),
                                                _dev(slot, "slot", I32), _dev(pos, "pos", I32), out.data_ptr(), T, H,
-                                               d, dr, r, S, float(scale), _stream()))
+                                               d, dr, r, S, float(scale), splits, _opt(part, "part", F32), _stream()))
+    return out
+
+
+def latent_attention_tiles(qc: torch.Tensor, proj: torch.Tensor, q_off: int, cache_c: torch.Tensor,
+                           cache_kr: torch.Tensor, sink: Optional[torch.Tensor], seq_start: torch.Tensor,
+                           seq_slot: torch.Tensor, seq_pos0: torch.Tensor, max_len: int, *, H: int, d: int, dr: int,
+                           r: int, scale: float) -> torch.Tensor:
+    """The prompt form of ``latent_attention``: tiles of 16 consecutive tokens of a sequence against key tiles of 16
+    cached rows on fp32 MFMA. ``max_len``: the most tokens any sequence brings to this step. r % 64 == 0."""
+    T, ld = proj.shape
+    B = seq_slot.numel()
+    S = cache_c.shape[1]
+    if qc.shape != (T, H * r) or (sink is not None and sink.numel() != H) or seq_start.numel() != B + 1:
+        raise ValueError("latent_attention_tiles: shapes")
+    out = torch.empty(T, H * r, dtype=F32, device=proj.device)
+    _check(load_library().lgs_latent_attention_tiles(
+        _dev(qc, "qc", F32), _dev(proj, "proj", F32), ld, q_off, _dev(cache_c, "cache_c"), _wf32(cache_c, "cache_c"),
+        _dev(cache_kr, "cache_kr", F32), _opt(sink, "sink", F32), _dev(seq_start, "seq_start", I32),
+        _dev(seq_slot, "seq_slot", I32), _dev(seq_pos0, "seq_pos0", I32), out.data_ptr(), B, int(max_len), H, d, dr, r,
+        S, float(scale), _stream()))
     return out
 
 
@@ -256,8 +283,9 @@ def moe_sort(ids: torch.Tensor, E: int):
     z_start = torch.empty(E + 1, dtype=I32, device=dev)
     tok_of = torch.empty(T * top, dtype=I32, device=dev)
     where = torch.empty(T * top, dtype=I32, device=dev)
+    ws = torch.zeros(2 * E, dtype=I32, device=dev)
     _check(load_library().lgs_moe_sort(_dev(ids, "ids", I32), T * top, top, E, z_start.data_ptr(), tok_of.data_ptr(),
-                                       where.data_ptr(), _stream()))
+                                       where.data_ptr(), ws.data_ptr(), _stream()))
     return z_start, tok_of, where
 
 

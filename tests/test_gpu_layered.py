@@ -48,7 +48,7 @@ def make_cfg(layers, width=48, vocab=61, loop=None, side=6, eps=1e-5, emb_scale=
     return cfg
 
 
-MIXED = [(ret(), dense()), (lat(), moe()), (ret(heads=3, dim=8, vdim=12, rot_dims=4), moe(top=1)), (lat(heads=3), None)]
+MIXED = [(ret(), dense()), (lat(), moe()), (ret(heads=3, dim=8, vdim=12, rot_dims=4), moe(top=1)), (lat(heads=3, kv_rank=64), None)]
 
 
 def build(cfg, dtype=torch.float32, seed=0):
@@ -118,6 +118,8 @@ TOL32, TOL16 = 2e-4, 6e-2
     ([(lat(), None)], 0),
     ([(lat(heads=1, dim=4, rot_dim=2, vdim=6, kv_rank=10), None)], 0),
     ([(lat(heads=3, dim=16, rot_dim=72, vdim=8, kv_rank=136), None)], 0),
+    ([(lat(heads=2, dim=8, rot_dim=6, vdim=8, kv_rank=64), None)], 0),
+    ([(lat(heads=2, dim=8, rot_dim=16, vdim=24, kv_rank=192), dense())], 0),
     ([(ret(), dense())], 0),
     ([(ret(), moe())], 0),
     ([(lat(), moe(ff=7, experts=1, top=1))], 0),
@@ -267,14 +269,14 @@ def test_far_key_and_sink_stand_out(cache_dtype):
 
     dev = torch.device("cuda", 0)
     g = torch.Generator().manual_seed(5)
-    H, d, dr, r, S = 2, 4, 6, 40, 704
+    H, d, dr, r, S = 2, 4, 6, 64, 704
     n = 700
     c = 0.1 * torch.randn(n, r, generator=g)
     kr = torch.randn(n, dr, generator=g)
     qc = torch.randn(H, r, generator=g) * 0.1
     qr = torch.randn(H, dr, generator=g) * 0.1
     c[3] = 0.5 * torch.sign(torch.randn(r, generator=g))
-    qc[0] = 4.0 * c[3]  # head 0: score 40 at row 3, about +-1.5 elsewhere
+    qc[0] = (160.0 / r) * c[3]  # head 0: score 40 at row 3, about +-1 elsewhere
     if cache_dtype == torch.bfloat16:
         c = c.to(torch.bfloat16).float()
     cache_c = torch.zeros(2, S, r, dtype=cache_dtype)
@@ -289,6 +291,12 @@ def test_far_key_and_sink_stand_out(cache_dtype):
                                            cache_c.to(dev), cache_kr.to(dev), sink.to(dev),
                                            torch.ones(T, dtype=torch.int32, device=dev), pos.to(dev), H=H, d=d, dr=dr,
                                            r=r, scale=1.0).cpu().view(T, H, r)
+            if T > 1:  # the same rows through the prompt form (one sequence in slot 1 that starts at n - T)
+                i32 = lambda *x: torch.tensor(x, dtype=torch.int32, device=dev)  # noqa: E731
+                tiles = seq_ops.latent_attention_tiles(qc.reshape(1, -1).repeat(T, 1).contiguous().to(dev), proj.to(dev), 0,
+                                                       cache_c.to(dev), cache_kr.to(dev), sink.to(dev), i32(0, T), i32(1),
+                                                       i32(n - T), T, H=H, d=d, dr=dr, r=r, scale=1.0).cpu().view(T, H, r)
+                assert (tiles - out).abs().max() < 1e-4 * max(1.0, float(out.abs().max()))
             for t in range(T):
                 L = int(pos[t]) + 1
                 for h in range(H):
@@ -401,10 +409,14 @@ def test_linear_per_head_and_grouped(T, wdtype):
     ids = torch.randint(0, E, (T, top), generator=g).to(torch.int32)
     z_start, tok_of, where = seq_ops.moe_sort(ids.cuda(), E)
     flat = ids.reshape(-1)
-    order = torch.sort(flat.long(), stable=True).indices
-    assert tok_of.cpu().tolist() == (order // top).tolist()
-    assert where.cpu()[order].tolist() == list(range(T * top))
     assert z_start.cpu().tolist() == [0] + torch.cumsum(torch.bincount(flat.long(), minlength=E), 0).tolist()
+    wh = where.cpu().long()
+    assert sorted(wh.tolist()) == list(range(T * top))  # a permutation ...
+    assert tok_of.cpu()[wh].tolist() == [i // top for i in range(T * top)]  # ... that remembers every pair's token
+    for e in range(E):  # ... and puts every pair into its expert's range
+        assert all(int(z_start[e]) <= int(w) < int(z_start[e + 1]) for w in wh[flat == e])
+    order = torch.empty(T * top, dtype=torch.long)
+    order[wh] = torch.arange(T * top)
     hmat = torch.randn(T, K, generator=g)
     we = torch.randn(E, N, K, generator=g).to(torch.bfloat16)
     out = torch.zeros(T * top, N).cuda()
