@@ -110,6 +110,9 @@ __global__ void __launch_bounds__(256) retention_chunk_kernel(RetArgs p) {
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int d = p.d, dv = p.dv, half = p.rot_dims / 2;
   const int DT = (d + 15) / 16, DPAD = DT * 16, DP = DPAD + 2;
+  int dshift = 4;
+  while ((1 << dshift) < DPAD) ++dshift;
+  const int DPOW = 1 << dshift;
   float* Qs = lds;
   float* Ks = Qs + kRC * DP;
   float* Vs = Ks + kRC * DP;
@@ -129,9 +132,9 @@ __global__ void __launch_bounds__(256) retention_chunk_kernel(RetArgs p) {
   for (int tc = t0; tc < t1; tc += kRC) {
     const int n = min(kRC, t1 - tc);
     // ---- load: q and k rotated (pairs dd, dd + half), k scaled; rows past n and dims past d are zero
-    for (int i = tid; i < kRC * DPAD; i += 256) {
-      const int row = i / DPAD, dd = i - row * DPAD;
-      if (dd >= half && dd < 2 * half) continue;  // written by its partner
+    for (int i = tid; i < kRC * DPOW; i += 256) {
+      const int row = i >> dshift, dd = i & (DPOW - 1);  // DPOW: DPAD rounded up to a power of two
+      if (dd >= DPAD || (dd >= half && dd < 2 * half)) continue;  // (rotated upper halves: written by the partner)
       const bool in = row < n && dd < d;
       const float* qr = p.q + (size_t)(tc + row) * p.ld + (size_t)h * d;
       const float* kr = p.k + (size_t)(tc + row) * p.ld + (size_t)h * d;
@@ -162,21 +165,32 @@ __global__ void __launch_bounds__(256) retention_chunk_kernel(RetArgs p) {
     __syncthreads();
     // ---- wave w owns tokens 16 w .. 16 w + 15: decayed causal scores, and the carried state's share of o
     const int ti = wave;
-    for (int tj = 0; tj < 4; ++tj) {
-      f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-      if (tj <= ti)
-        for (int k = 0; k < DPAD; k += 4)
-          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(Qs[(ti * 16 + fr) * DP + k + fk], Ks[(tj * 16 + fr) * DP + k + fk],
-                                                     acc, 0, 0, 0);
+    {
+      // the four key blocks as independent chains (blocks right of the diagonal are skipped and left zero)
+      f32x4_t acc[4];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int i = ti * 16 + fk * 4 + r, j = tj * 16 + fr;
-        As[i * kAS + j] = j <= i ? acc[r] * pw[i - j] : 0.0f;
+      for (int tj = 0; tj < 4; ++tj) acc[tj] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      const float* qa = Qs + (ti * 16 + fr) * DP + fk;
+      const float* kb = Ks + fr * DP + fk;
+#pragma unroll 2
+      for (int k = 0; k < DPAD; k += 4) {
+        const float a = qa[k];
+#pragma unroll
+        for (int tj = 0; tj < 4; ++tj)
+          if (tj <= ti) acc[tj] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, kb[tj * 16 * DP + k], acc[tj], 0, 0, 0);
       }
+#pragma unroll
+      for (int tj = 0; tj < 4; ++tj)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int i = ti * 16 + fk * 4 + r, j = tj * 16 + fr;
+          As[i * kAS + j] = j <= i ? acc[tj][r] * pw[i - j] : 0.0f;
+        }
     }
     f32x4_t o[4];
 #pragma unroll
     for (int c = 0; c < 4; ++c) o[c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
     for (int k = 0; k < DPAD; k += 4) {
       const float a = Qs[(ti * 16 + fr) * DP + k + fk];
 #pragma unroll
@@ -189,6 +203,7 @@ __global__ void __launch_bounds__(256) retention_chunk_kernel(RetArgs p) {
       for (int r = 0; r < 4; ++r) o[c][r] *= pw[ti * 16 + fk * 4 + r + 1];
     __syncthreads();
     // ---- o += scores . V (keys up to the wave's last token), then out
+#pragma unroll 4
     for (int k = 0; k < (ti + 1) * 16; k += 4) {
       const float a = As[(ti * 16 + fr) * kAS + k + fk];
 #pragma unroll
@@ -210,6 +225,7 @@ __global__ void __launch_bounds__(256) retention_chunk_kernel(RetArgs p) {
       for (int c = 0; c < 4; ++c)
 #pragma unroll
         for (int r = 0; r < 4; ++r) s[c][r] = pn * Ss[(td * 16 + fk * 4 + r) * kVS + c * 16 + fr];
+#pragma unroll 4
       for (int k = 0; k < kRC; k += 4) {
         const int j = k + fk;
         const float a = j < n ? Ks[j * DP + td * 16 + fr] * pw[n - 1 - j] : 0.0f;
@@ -422,8 +438,10 @@ __global__ void __launch_bounds__(256) latent_attention_kernel(LatAttArgs p, flo
 // The prompt form: 16 consecutive tokens of one sequence and one head per workgroup, key tiles of 16 cached rows
 // staged in LDS as fp32, both products on v_mfma_f32_16x16x4_f32. The four waves split the score product over the
 // latent / rotated dims (partial 16x16 tiles summed through LDS) and the weighted sum over the r output columns
-// (NT tiles of 16 per wave); each runs the same online softmax on the summed scores. The next key tile travels in
-// registers while the current one is multiplied. r % 64 == 0.
+// (NT tiles of 16 per wave); each runs the same online softmax on the summed scores. A wave keeps its share of the
+// 16 queries in registers (one value per lane and score instruction), so LDS holds the key tile only and three
+// workgroups fit a CU. The next key tile travels in registers while the current one is multiplied; the longest
+// tiles (the sequence's last tokens) are launched first. r % 64 == 0.
 struct LatTileArgs {
   LatAttArgs a;
   const int* seq_start;
@@ -436,75 +454,82 @@ __global__ void __launch_bounds__(256) latent_attention_tile_kernel(LatTileArgs 
   extern __shared__ float lds[];
   const LatAttArgs& p = tp.a;
   const int b = blockIdx.z, h = blockIdx.y;
-  const int t0 = tp.seq_start[b] + blockIdx.x * 16, t1 = tp.seq_start[b + 1];
+  const int tile = gridDim.x - 1 - blockIdx.x;
+  const int t0 = tp.seq_start[b] + tile * 16, t1 = tp.seq_start[b + 1];
   if (t0 >= t1) return;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, fr = lane & 15, fk = lane >> 4;
   const int r = p.r, dr = p.dr, D = r + dr;
   const int DQ = (D + 15) / 16 * 4;             // dims per wave in the score product (multiple of 4)
   const int KP = (4 * DQ + 31) / 32 * 32 + 2;   // row stride of the Q and key tiles (conflict-free 16 x 4 reads)
-  float* Qt = lds;                  // [16][KP]
-  float* Kt = Qt + 16 * KP;         // [16][KP]
+  float* Kt = lds;                  // [16][KP]
   float* Sp = Kt + 16 * KP;         // [4][16][17] partial scores
   float* Pw = Sp + 4 * 16 * 17;     // [4][16][17] each wave's copy of the weights
   const int rows = min(16, t1 - t0);
-  const int pos_first = tp.seq_pos0[b] + blockIdx.x * 16;
+  const int pos_first = tp.seq_pos0[b] + tile * 16;
   const int pos_last = min(pos_first + rows - 1, p.max_seq - 1);
   const size_t base = (size_t)tp.seq_slot[b] * p.max_seq;
-  for (int i = tid; i < 16 * KP; i += 256) {
-    const int row = i / KP, dd = i - row * KP;
+  // this lane's query operands: row fr, dims wave DQ + fk + 4 i (the latent part, then the rotated part, then zeros)
+  constexpr int NQ = 40;  // (512 + 128) / 16
+  float qreg[NQ];
+#pragma unroll
+  for (int i = 0; i < NQ; ++i) {
+    const int dd = wave * DQ + fk + 4 * i;
     float v = 0.0f;
-    if (row < rows) {
-      if (dd < r) v = p.qc[((size_t)(t0 + row) * p.H + h) * r + dd];
-      else if (dd < D) v = p.proj[(size_t)(t0 + row) * p.ld + p.q_off + (size_t)h * (p.d + dr) + p.d + (dd - r)];
+    if (4 * i < DQ && fr < rows) {
+      if (dd < r) v = p.qc[((size_t)(t0 + fr) * p.H + h) * r + dd];
+      else if (dd < D) v = p.proj[(size_t)(t0 + fr) * p.ld + p.q_off + (size_t)h * (p.d + dr) + p.d + (dd - r)];
     }
-    Qt[i] = v;
-    Kt[i] = 0.0f;  // the padding columns stay zero; the live ones are rewritten per tile
+    qreg[i] = v;
   }
+  for (int i = tid; i < 16 * KP; i += 256) Kt[i] = 0.0f;  // the padding columns stay zero
   constexpr int NC = CF32 ? 8 : 4;  // 16-B loads of the latent part per thread (r <= 512)
   uint4 creg[NC];
   float kreg[8];
   const int cvec = CF32 ? r / 4 : r / 8;  // 16-B vectors per cached latent row
+  // which key of a tile, and which part of its row, each of this thread's loads covers (fixed for the whole kernel:
+  // no integer division inside the tile loop); key -1 marks a load this thread does not have
+  int ckey[NC], coff[NC], kkey[8], koff[8];
+#pragma unroll
+  for (int i = 0; i < NC; ++i) {
+    const int idx = tid + 256 * i;
+    ckey[i] = idx < 16 * cvec ? idx / cvec : -1;
+    coff[i] = (idx % cvec) * (CF32 ? 4 : 8);
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int idx = tid + 256 * i;
+    kkey[i] = idx < 16 * dr ? idx / dr : -1;
+    koff[i] = dr ? idx % dr : 0;
+  }
   auto gload = [&](int kt) {
 #pragma unroll
-    for (int i = 0; i < NC; ++i) {
-      const int idx = tid + 256 * i;
-      if (idx < 16 * cvec) {
-        const int key = min(kt * 16 + idx / cvec, p.max_seq - 1), v = idx % cvec;
-        creg[i] = CF32 ? ((const uint4*)((const float*)p.cache_c + (base + key) * r))[v]
-                       : ((const uint4*)((const uint16_t*)p.cache_c + (base + key) * r))[v];
+    for (int i = 0; i < NC; ++i)
+      if (ckey[i] >= 0) {
+        const size_t row = base + min(kt * 16 + ckey[i], p.max_seq - 1);
+        creg[i] = CF32 ? *(const uint4*)((const float*)p.cache_c + row * r + coff[i])
+                       : *(const uint4*)((const uint16_t*)p.cache_c + row * r + coff[i]);
       }
-    }
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int idx = tid + 256 * i;
-      if (idx < 16 * dr) kreg[i] = p.cache_kr[(base + min(kt * 16 + idx / dr, p.max_seq - 1)) * dr + idx % dr];
-    }
+    for (int i = 0; i < 8; ++i)
+      if (kkey[i] >= 0) kreg[i] = p.cache_kr[(base + min(kt * 16 + kkey[i], p.max_seq - 1)) * dr + koff[i]];
   };
   auto lstore = [&]() {
 #pragma unroll
-    for (int i = 0; i < NC; ++i) {
-      const int idx = tid + 256 * i;
-      if (idx < 16 * cvec) {
-        const int key = idx / cvec, v = idx % cvec;
-        float* dst = Kt + key * KP + v * (CF32 ? 4 : 8);
+    for (int i = 0; i < NC; ++i)
+      if (ckey[i] >= 0) {
+        float* dst = Kt + ckey[i] * KP + coff[i];
         const uint32_t w[4] = {creg[i].x, creg[i].y, creg[i].z, creg[i].w};
-        if (CF32) {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) dst[e] = __uint_as_float(w[e]);
+        if (CF32) {  // (rows are 8-byte aligned: KP is even)
+          ((float2*)dst)[0] = make_float2(__uint_as_float(w[0]), __uint_as_float(w[1]));
+          ((float2*)dst)[1] = make_float2(__uint_as_float(w[2]), __uint_as_float(w[3]));
         } else {
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            dst[2 * e] = bflo(w[e]);
-            dst[2 * e + 1] = bfhi(w[e]);
-          }
+          for (int e = 0; e < 4; ++e) ((float2*)dst)[e] = make_float2(bflo(w[e]), bfhi(w[e]));
         }
       }
-    }
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int idx = tid + 256 * i;
-      if (idx < 16 * dr) Kt[(idx / dr) * KP + r + idx % dr] = kreg[i];
-    }
+    for (int i = 0; i < 8; ++i)
+      if (kkey[i] >= 0) Kt[kkey[i] * KP + r + koff[i]] = kreg[i];
   };
   f32x4_t o[NT];
 #pragma unroll
@@ -519,16 +544,25 @@ __global__ void __launch_bounds__(256) latent_attention_tile_kernel(LatTileArgs 
   }
   const int nkt = pos_last / 16 + 1;
   gload(0);
-  __syncthreads();  // Qt, and Kt's zero padding
+  __syncthreads();  // Kt's zero padding
   for (int kt = 0; kt < nkt; ++kt) {
     lstore();
     __syncthreads();
     if (kt + 1 < nkt) gload(kt + 1);
     // partial scores over this wave's dims
-    f32x4_t sacc = {0.f, 0.f, 0.f, 0.f};
-    const float* qa = Qt + fr * KP + wave * DQ + fk;
+    // (four independent chains, so that LDS reads and matrix instructions overlap)
+    f32x4_t sacc = {0.f, 0.f, 0.f, 0.f}, s1 = sacc, s2 = sacc, s3 = sacc;
     const float* kb = Kt + fr * KP + wave * DQ + fk;
-    for (int k = 0; k < DQ; k += 4) sacc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[k], kb[k], sacc, 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < NQ; i += 4) {
+      if (4 * i >= DQ) break;
+      sacc = __builtin_amdgcn_mfma_f32_16x16x4f32(qreg[i], kb[4 * i], sacc, 0, 0, 0);
+      if (4 * (i + 1) < DQ) s1 = __builtin_amdgcn_mfma_f32_16x16x4f32(qreg[i + 1], kb[4 * i + 4], s1, 0, 0, 0);
+      if (4 * (i + 2) < DQ) s2 = __builtin_amdgcn_mfma_f32_16x16x4f32(qreg[i + 2], kb[4 * i + 8], s2, 0, 0, 0);
+      if (4 * (i + 3) < DQ) s3 = __builtin_amdgcn_mfma_f32_16x16x4f32(qreg[i + 3], kb[4 * i + 12], s3, 0, 0, 0);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sacc[j] = (sacc[j] + s1[j]) + (s2[j] + s3[j]);
 #pragma unroll
     for (int j = 0; j < 4; ++j) Sp[(wave * 16 + fk * 4 + j) * 17 + fr] = sacc[j];
     __syncthreads();
@@ -700,7 +734,7 @@ extern "C" int lgs_latent_attention_tiles(const float* qc, const float* proj, lo
   lgs::LatTileArgs p{{qc, proj, ld, q_off, cache_c, cache_kr, sink, nullptr, nullptr, out, H, d, dr, r, max_seq, scale},
                      seq_start, seq_slot, seq_pos0};
   const int D = r + dr, DQ = (D + 15) / 16 * 4, KP = (4 * DQ + 31) / 32 * 32 + 2;
-  const size_t lds = (size_t)(2 * 16 * KP + 2 * 4 * 16 * 17) * sizeof(float);
+  const size_t lds = (size_t)(16 * KP + 2 * 4 * 16 * 17) * sizeof(float);
   const dim3 grid((max_len + 15) / 16, H, B);
   const void* fn = nullptr;
 #define LGS_TILE(NT)                                                                                   \
