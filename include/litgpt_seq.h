@@ -50,10 +50,15 @@ int lgs_gather_rows(const float* x, const int* rows, float* y, int n_rows, int W
 /* retention: rotary (pairs i, i + rot_dims/2; angle = position * inv_freq[i]) on q and k, k * k_scale, then per
  * sequence and head S <- decay S + k v^T, o = S^T q. state [slots][H][d][dv] fp32 is read unless the sequence's
  * first position is 0 and written back at the end of the step. d <= 256. chunked != 0 (and d <= 128) runs the
- * prompt form: chunks of 64 tokens as fp32 matrix products, the state carried from chunk to chunk in LDS. */
-int lgs_retention(const float* q, const float* k, const float* v, long ld, float* state, const float* decay,
+ * prompt form: chunks of 64 tokens as fp32 matrix products, the state carried from chunk to chunk in LDS; with a
+ * workspace ws of B * max_chunks * H * d * dv floats (max_chunks = 64-token chunks of the longest sequence) the chunks
+ * run side by side when sequences and heads alone would not fill the chip: local sums, a short carry over the
+ * chunks, then the outputs. The prompt form rotates and scales q and k IN PLACE first (T_rows rows with positions
+ * pos[T_rows]); the token-by-token form leaves them as they are. */
+int lgs_retention(float* q, float* k, const float* v, long ld, float* state, const float* decay,
                   const float* inv_freq, const int* seq_start, const int* seq_slot, const int* seq_pos0, float* out,
-                  int B, int H, int d, int dv, int rot_dims, float k_scale, int chunked, lgs_stream_t stream);
+                  int B, int H, int d, int dv, int rot_dims, float k_scale, int chunked, float* ws, int max_chunks,
+                  int T_rows, const int* pos, lgs_stream_t stream);
 /* in place on o [T][H][dv]: (unit_norm ? o / rms(o) per head : o) * act(g[t * ldg + h * dv + i]) */
 int lgs_head_gate(float* o, const float* g, long ldg, int T, int H, int dv, int unit_norm, float eps, int act,
                   lgs_stream_t stream);

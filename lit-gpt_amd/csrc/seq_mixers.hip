@@ -29,6 +29,8 @@ struct RetArgs {
   float* out;            // [T][H * dv]
   int H, d, dv, rot_dims;
   float k_scale;
+  float* ws;       // chunk-parallel prompt form: [B * max_chunks][H][d][dv] local sums, then chunk-start states
+  int max_chunks;  // chunks of 64 tokens of the longest sequence
 };
 
 // grid (B, H, ceil(dv / 64)): a workgroup owns 64 columns of one head's state; wave w owns rows [w NR, (w + 1) NR)
@@ -99,17 +101,49 @@ __global__ void __launch_bounds__(256) retention_scan_kernel(RetArgs p) {
 // The prompt form: the same recurrence over chunks of 64 tokens as fp32 matrix products (v_mfma_f32_16x16x4_f32).
 // With S the state at the chunk's start, n its token count and i, j local positions:
 //   o_i = decay^(i+1) S^T q_i + sum_{j <= i} decay^(i-j) (q_i . k_j) v_j,   S' = decay^n S + sum_j decay^(n-1-j) k_j v_j^T
-// grid (B, H, ceil(dv / 64)); a workgroup keeps 64 columns of the state in LDS and walks its sequence's chunks.
+// MODE 0, grid (B, H, ceil(dv / 64)): a workgroup keeps 64 columns of the state in LDS and walks its sequence's
+// chunks one after the other. With a workspace the chunks run side by side instead, grid (B * max_chunks, H, ..):
+// MODE 1 leaves every chunk's local sum (the second term of S') in the workspace, retention_carry_kernel turns these
+// into the state at each chunk's start (a short elementwise recurrence over the chunks, which also leaves the final
+// state), and MODE 2 computes the outputs of every chunk from its start state.
 // LDS (floats): Q, K [64][DP], V [64][80], scores [64][66], S [DPAD][80], powers of the decay [66]; d <= 128.
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 constexpr int kRC = 64, kVS = 80, kAS = 66;
 
+// grid (T, H): rotary on q and k in place (pairs i, i + rot_dims / 2) and the key scale, ahead of the chunk kernels
+__global__ void __launch_bounds__(64) retention_rope_kernel(float* __restrict__ q, float* __restrict__ k, long ld,
+                                                            const float* __restrict__ inv_freq,
+                                                            const int* __restrict__ pos, int d, int rot_dims,
+                                                            float k_scale) {
+  const int t = blockIdx.x, h = blockIdx.y, half = rot_dims / 2;
+  float* qr = q + (size_t)t * ld + (size_t)h * d;
+  float* kr = k + (size_t)t * ld + (size_t)h * d;
+  const float fpos = (float)pos[t];
+  for (int i = threadIdx.x; i < d; i += 64) {
+    if (i < half) {
+      float sn, cs;
+      sincosf(fpos * inv_freq[i], &sn, &cs);
+      const float qu = qr[i], qv = qr[i + half], ku = kr[i], kv = kr[i + half];
+      qr[i] = qu * cs - qv * sn;
+      qr[i + half] = qv * cs + qu * sn;
+      kr[i] = (ku * cs - kv * sn) * k_scale;
+      kr[i + half] = (kv * cs + ku * sn) * k_scale;
+    } else if (i >= rot_dims) {
+      kr[i] *= k_scale;
+    }
+  }
+}
+
+// DPC: the key dim padded to 16 when it is 64 or 128 (constant trip counts), 0 for any other
+template <int MODE, int DPC>
 __global__ void __launch_bounds__(256) retention_chunk_kernel(RetArgs p) {
   extern __shared__ float lds[];
-  const int b = blockIdx.x, h = blockIdx.y, col0 = blockIdx.z * 64;
+  const int b = MODE == 0 ? blockIdx.x : blockIdx.x / p.max_chunks;
+  const int cidx = MODE == 0 ? 0 : blockIdx.x % p.max_chunks;
+  const int h = blockIdx.y, col0 = blockIdx.z * 64;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const int d = p.d, dv = p.dv, half = p.rot_dims / 2;
-  const int DT = (d + 15) / 16, DPAD = DT * 16, DP = DPAD + 2;
+  const int d = p.d, dv = p.dv;
+  const int DPAD = DPC ? DPC : (d + 15) / 16 * 16, DT = DPAD / 16, DP = DPAD + 2;
   int dshift = 4;
   while ((1 << dshift) < DPAD) ++dshift;
   const int DPOW = 1 << dshift;
@@ -120,43 +154,30 @@ __global__ void __launch_bounds__(256) retention_chunk_kernel(RetArgs p) {
   float* Ss = As + kRC * kAS;
   float* pw = Ss + DPAD * kVS;
   const int t0 = p.seq_start[b], t1 = p.seq_start[b + 1];
+  if (MODE != 0 && t0 + cidx * kRC >= t1) return;
   const int pos0 = p.seq_pos0[b];
   const float lam = p.decay[h];
-  float* sp = p.state + (((size_t)p.seq_slot[b] * p.H + h) * d) * dv;
-  for (int i = tid; i < DPAD * 64; i += 256) {
-    const int row = i >> 6, c = i & 63;
-    Ss[row * kVS + c] = (pos0 > 0 && row < d && col0 + c < dv) ? sp[(size_t)row * dv + col0 + c] : 0.0f;
-  }
+  // MODE 0: the slot's state; MODE 1 / 2: this chunk's tile of the workspace
+  float* sp = MODE == 0 ? p.state + (((size_t)p.seq_slot[b] * p.H + h) * d) * dv
+                        : p.ws + (((size_t)blockIdx.x * p.H + h) * d) * dv;
+  if (MODE != 1)
+    for (int i = tid; i < DPAD * 64; i += 256) {
+      const int row = i >> 6, c = i & 63;
+      Ss[row * kVS + c] = ((MODE == 2 || pos0 > 0) && row < d && col0 + c < dv) ? sp[(size_t)row * dv + col0 + c] : 0.0f;
+    }
   if (tid <= 64) pw[tid] = powf(lam, (float)tid);
   const int fr = lane & 15, fk = lane >> 4;
-  for (int tc = t0; tc < t1; tc += kRC) {
+  const int t_end = MODE == 0 ? t1 : min(t1, t0 + (cidx + 1) * kRC);
+  for (int tc = t0 + cidx * kRC; tc < t_end; tc += kRC) {
     const int n = min(kRC, t1 - tc);
-    // ---- load: q and k rotated (pairs dd, dd + half), k scaled; rows past n and dims past d are zero
+    // ---- load (q and k were rotated and scaled in place beforehand); rows past n and dims past d are zero
     for (int i = tid; i < kRC * DPOW; i += 256) {
-      const int row = i >> dshift, dd = i & (DPOW - 1);  // DPOW: DPAD rounded up to a power of two
-      if (dd >= DPAD || (dd >= half && dd < 2 * half)) continue;  // (rotated upper halves: written by the partner)
+      const int row = i >> dshift, dd = i & (DPOW - 1);
+      if (dd >= DPAD) continue;
       const bool in = row < n && dd < d;
-      const float* qr = p.q + (size_t)(tc + row) * p.ld + (size_t)h * d;
-      const float* kr = p.k + (size_t)(tc + row) * p.ld + (size_t)h * d;
-      if (dd < half) {
-        float q0 = 0.f, q1 = 0.f, k0 = 0.f, k1 = 0.f;
-        if (row < n) {
-          float sn, cs;
-          sincosf((float)(pos0 + (tc - t0) + row) * p.inv_freq[dd], &sn, &cs);
-          const float qu = qr[dd], qv = qr[dd + half], ku = kr[dd], kv = kr[dd + half];
-          q0 = qu * cs - qv * sn;
-          q1 = qv * cs + qu * sn;
-          k0 = (ku * cs - kv * sn) * p.k_scale;
-          k1 = (kv * cs + ku * sn) * p.k_scale;
-        }
-        Qs[row * DP + dd] = q0;
-        Qs[row * DP + dd + half] = q1;
-        Ks[row * DP + dd] = k0;
-        Ks[row * DP + dd + half] = k1;
-      } else {
-        Qs[row * DP + dd] = in ? qr[dd] : 0.0f;
-        Ks[row * DP + dd] = in ? kr[dd] * p.k_scale : 0.0f;
-      }
+      const size_t at = (size_t)(tc + row) * p.ld + (size_t)h * d + dd;
+      if (MODE != 1) Qs[row * DP + dd] = in ? p.q[at] : 0.0f;
+      Ks[row * DP + dd] = in ? p.k[at] : 0.0f;
     }
     for (int i = tid; i < kRC * 64; i += 256) {
       const int row = i >> 6, c = i & 63;
@@ -165,7 +186,7 @@ __global__ void __launch_bounds__(256) retention_chunk_kernel(RetArgs p) {
     __syncthreads();
     // ---- wave w owns tokens 16 w .. 16 w + 15: decayed causal scores, and the carried state's share of o
     const int ti = wave;
-    {
+    if (MODE != 1) {
       // the four key blocks as independent chains (blocks right of the diagonal are skipped and left zero)
       f32x4_t acc[4];
 #pragma unroll
@@ -186,7 +207,6 @@ __global__ void __launch_bounds__(256) retention_chunk_kernel(RetArgs p) {
           const int i = ti * 16 + fk * 4 + r, j = tj * 16 + fr;
           As[i * kAS + j] = j <= i ? acc[tj][r] * pw[i - j] : 0.0f;
         }
-    }
     f32x4_t o[4];
 #pragma unroll
     for (int c = 0; c < 4; ++c) o[c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -217,14 +237,15 @@ __global__ void __launch_bounds__(256) retention_chunk_kernel(RetArgs p) {
         const int i = ti * 16 + fk * 4 + r, col = col0 + c * 16 + fr;
         if (i < n && col < dv) p.out[(size_t)(tc + i) * p.H * dv + (size_t)h * dv + col] = o[c][r];
       }
+    }
     // ---- state: S' = decay^n S + sum_j decay^(n-1-j) k_j v_j^T; each element of S belongs to one lane
     const float pn = pw[n];
-    for (int td = wave; td < DT; td += 4) {
+    for (int td = wave; td < DT && MODE != 2; td += 4) {
       f32x4_t s[4];
 #pragma unroll
       for (int c = 0; c < 4; ++c)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) s[c][r] = pn * Ss[(td * 16 + fk * 4 + r) * kVS + c * 16 + fr];
+        for (int r = 0; r < 4; ++r) s[c][r] = MODE == 1 ? 0.0f : pn * Ss[(td * 16 + fk * 4 + r) * kVS + c * 16 + fr];
 #pragma unroll 4
       for (int k = 0; k < kRC; k += 4) {
         const int j = k + fk;
@@ -236,14 +257,41 @@ __global__ void __launch_bounds__(256) retention_chunk_kernel(RetArgs p) {
 #pragma unroll
       for (int c = 0; c < 4; ++c)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) Ss[(td * 16 + fk * 4 + r) * kVS + c * 16 + fr] = s[c][r];
+        for (int r = 0; r < 4; ++r) {
+          const int row = td * 16 + fk * 4 + r, col = c * 16 + fr;
+          if (MODE == 0) Ss[row * kVS + col] = s[c][r];
+          else if (row < d && col0 + col < dv) sp[(size_t)row * dv + col0 + col] = s[c][r];
+        }
     }
     __syncthreads();
   }
-  for (int i = tid; i < DPAD * 64; i += 256) {
-    const int row = i >> 6, c = i & 63;
-    if (row < d && col0 + c < dv) sp[(size_t)row * dv + col0 + c] = Ss[row * kVS + c];
+  if (MODE == 0)
+    for (int i = tid; i < DPAD * 64; i += 256) {
+      const int row = i >> 6, c = i & 63;
+      if (row < d && col0 + c < dv) sp[(size_t)row * dv + col0 + c] = Ss[row * kVS + c];
+    }
+}
+
+// grid (B, H, ceil(d dv / 256)): one state element per thread walks its sequence's chunks: the workspace's local
+// sums become the states at the chunks' starts, and the state after the last chunk goes back to the slot
+__global__ void __launch_bounds__(256) retention_carry_kernel(RetArgs p) {
+  const int b = blockIdx.x, h = blockIdx.y;
+  const int e = blockIdx.z * 256 + threadIdx.x;
+  if (e >= p.d * p.dv) return;
+  const int len = p.seq_start[b + 1] - p.seq_start[b];
+  const float lam = p.decay[h];
+  const float p64 = powf(lam, (float)kRC);
+  float* sp = p.state + ((size_t)p.seq_slot[b] * p.H + h) * p.d * p.dv + e;
+  float S = p.seq_pos0[b] > 0 ? *sp : 0.0f;
+  const int chunks = (len + kRC - 1) / kRC;
+  for (int c = 0; c < chunks; ++c) {
+    float* w = p.ws + (((size_t)b * p.max_chunks + c) * p.H + h) * p.d * p.dv + e;
+    const float u = *w;
+    *w = S;
+    const int n = min(kRC, len - c * kRC);
+    S = fmaf(n == kRC ? p64 : powf(lam, (float)n), S, u);
   }
+  *sp = S;
 }
 
 static size_t retention_chunk_lds(int d) {
@@ -410,6 +458,107 @@ __global__ void __launch_bounds__(256) latent_attention_kernel(LatAttArgs p, flo
 #pragma unroll
   for (int e = 0; e < NR; ++e)
     if (lane + 64 * e < r) sacc[wave * r + lane + 64 * e] = acc[e];
+  __syncthreads();
+  const bool fin = splits == 1;
+  const float snk = (fin && p.sink) ? p.sink[h] : -INFINITY;
+  const float mx = fmaxf(fmaxf(fmaxf(sm[0], sm[1]), fmaxf(sm[2], sm[3])), snk);
+  float f[4], den = (fin && p.sink) ? expf(snk - mx) : 0.0f;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    f[w] = sl[w] > 0.0f ? expf(sm[w] - mx) : 0.0f;
+    den += sl[w] * f[w];
+  }
+  if (fin) {
+    float* o = p.out + ((size_t)t * p.H + h) * r;
+    for (int i = threadIdx.x; i < r; i += 256)
+      o[i] = ((sacc[i] * f[0] + sacc[r + i] * f[1]) + (sacc[2 * r + i] * f[2] + sacc[3 * r + i] * f[3])) / den;
+  } else {
+    float* o = part + (((size_t)t * p.H + h) * splits + z) * (r + 2);
+    if (threadIdx.x == 0) {
+      o[0] = mx;
+      o[1] = den;
+    }
+    for (int i = threadIdx.x; i < r; i += 256)
+      o[2 + i] = (sacc[i] * f[0] + sacc[r + i] * f[1]) + (sacc[2 * r + i] * f[2] + sacc[3 * r + i] * f[3]);
+  }
+}
+
+// The same walk with 16-byte loads: lane holds the 8 consecutive latent dims 8 lane .. 8 lane + 7 (r % 8 == 0,
+// r <= 512), so a cached row is one load instruction per wave instead of r / 64.
+template <bool CF32>
+__global__ void __launch_bounds__(256) latent_attention_vec_kernel(LatAttArgs p, float* __restrict__ part) {
+  __shared__ float sm[4], sl[4];
+  extern __shared__ float sacc[];  // [4][r]
+  constexpr int U = 4;
+  const int t = blockIdx.x, h = blockIdx.y, z = blockIdx.z, splits = gridDim.z;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r = p.r, dr = p.dr;
+  const int last = min(p.pos[t], p.max_seq - 1);
+  const int share = (last + splits) / splits;
+  const int lo = z * share, hi = min(last, lo + share - 1);
+  const size_t base = (size_t)p.slot[t] * p.max_seq;
+  const bool live = 8 * lane < r;
+  const float* qc = p.qc + ((size_t)t * p.H + h) * r + 8 * lane;
+  const float* qr = p.proj + (size_t)t * p.ld + p.q_off + (size_t)h * (p.d + dr) + p.d;
+  float q[8], qrot[2], acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    q[e] = live ? qc[e] : 0.0f;
+    acc[e] = 0.0f;
+  }
+#pragma unroll
+  for (int e = 0; e < 2; ++e) qrot[e] = lane + 64 * e < dr ? qr[lane + 64 * e] : 0.0f;
+  float m = -INFINITY, l = 0.0f;
+  for (int j0 = lo + wave; j0 <= hi; j0 += 4 * U) {
+    float c[U][8], dot[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int j = min(j0 + 4 * u, hi);
+      if (!live) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) c[u][e] = 0.0f;
+      } else if (CF32) {
+        const float4 a = *(const float4*)((const float*)p.cache_c + (base + j) * r + 8 * lane);
+        const float4 b = *(const float4*)((const float*)p.cache_c + (base + j) * r + 8 * lane + 4);
+        c[u][0] = a.x; c[u][1] = a.y; c[u][2] = a.z; c[u][3] = a.w;
+        c[u][4] = b.x; c[u][5] = b.y; c[u][6] = b.z; c[u][7] = b.w;
+      } else {
+        const uint4 w = *(const uint4*)((const uint16_t*)p.cache_c + (base + j) * r + 8 * lane);
+        c[u][0] = bflo(w.x); c[u][1] = bfhi(w.x); c[u][2] = bflo(w.y); c[u][3] = bfhi(w.y);
+        c[u][4] = bflo(w.z); c[u][5] = bfhi(w.z); c[u][6] = bflo(w.w); c[u][7] = bfhi(w.w);
+      }
+      dot[u] = 0.0f;
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const int i = lane + 64 * e;
+        if (i < dr) dot[u] = fmaf(qrot[e], p.cache_kr[(base + j) * dr + i], dot[u]);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) dot[u] = fmaf(q[e], c[u][e], dot[u]);
+      dot[u] = wave_sum(dot[u]) * p.scale;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (j0 + 4 * u > hi) break;
+      const float mn = fmaxf(m, dot[u]);
+      const float corr = expf(m - mn), w = expf(dot[u] - mn);
+      l = l * corr + w;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = acc[e] * corr + w * c[u][e];
+      m = mn;
+    }
+  }
+  if (lane == 0) {
+    sm[wave] = m;
+    sl[wave] = l;
+  }
+  if (live) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) sacc[wave * r + 8 * lane + e] = acc[e];
+  }
   __syncthreads();
   const bool fin = splits == 1;
   const float snk = (fin && p.sink) ? p.sink[h] : -INFINITY;
@@ -643,28 +792,50 @@ __global__ void __launch_bounds__(256) latent_combine_kernel(const float* __rest
 
 }  // namespace lgs
 
-extern "C" int lgs_retention(const float* q, const float* k, const float* v, long ld, float* state, const float* decay,
+extern "C" int lgs_retention(float* q, float* k, const float* v, long ld, float* state, const float* decay,
                              const float* inv_freq, const int* seq_start, const int* seq_slot, const int* seq_pos0,
                              float* out, int B, int H, int d, int dv, int rot_dims, float k_scale, int chunked,
-                             hipStream_t stream) {
+                             float* ws, int max_chunks, int T_rows, const int* pos, hipStream_t stream) {
   LGA_CHECK_ARG(q && k && v && state && decay && seq_start && seq_slot && seq_pos0 && out, "lgs_retention: null pointer");
   LGA_CHECK_ARG(B > 0 && H > 0 && H <= 65535 && d > 0 && d <= 256 && dv > 0, "lgs_retention: head dim must be in [1, 256]");
   LGA_CHECK_ARG(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= d && (rot_dims == 0 || inv_freq),
                 "lgs_retention: bad rotary dims");
-  lgs::RetArgs p{q, k, v, ld, state, decay, inv_freq, seq_start, seq_slot, seq_pos0, out, H, d, dv, rot_dims, k_scale};
+  LGA_CHECK_ARG(!ws || max_chunks > 0, "lgs_retention: a workspace needs the longest sequence's chunk count");
+  lgs::RetArgs p{q, k, v, ld, state, decay, inv_freq, seq_start, seq_slot, seq_pos0, out, H, d, dv, rot_dims, k_scale,
+                 ws, max_chunks};
   const dim3 grid(B, H, (dv + 63) / 64);
   if (chunked && d <= 128) {  // a prompt: chunks of 64 tokens as fp32 matrix products
+    LGA_CHECK_ARG(T_rows > 0 && pos, "lgs_retention: the prompt form needs the row count and the rows' positions");
+    if (rot_dims > 0 || k_scale != 1.0f)
+      lgs::retention_rope_kernel<<<dim3(T_rows, H), 64, 0, stream>>>((float*)q, (float*)k, ld, inv_freq, pos, d, rot_dims,
+                                                                     k_scale);
     const size_t lds = lgs::retention_chunk_lds(d);
-    static size_t allowed = 0;
-    if (lds > allowed) {
-      if (hipFuncSetAttribute((const void*)lgs::retention_chunk_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                              (int)lds) != hipSuccess) {
-        lga_set_error("lgs_retention: cannot reserve the chunk kernel's LDS");
-        return (int)hipErrorInvalidValue;
-      }
-      allowed = lds;
+    const bool side = ws && (long)B * H * ((dv + 63) / 64) < lga::num_cu() && (long)B * max_chunks <= 1 << 24;
+    const dim3 cgrid(side ? B * max_chunks : B, H, (dv + 63) / 64);
+#define LGS_RET(MODE, DPC, G)                                                                                          \
+  do {                                                                                                                 \
+    if (hipFuncSetAttribute((const void*)lgs::retention_chunk_kernel<MODE, DPC>,                                       \
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {                     \
+      lga_set_error("lgs_retention: cannot reserve the chunk kernel's LDS");                                           \
+      return (int)hipErrorInvalidValue;                                                                                \
+    }                                                                                                                  \
+    lgs::retention_chunk_kernel<MODE, DPC><<<G, 256, lds, stream>>>(p);                                                \
+  } while (0)
+#define LGS_RET_D(MODE, G)              \
+  do {                                  \
+    if (d == 128) LGS_RET(MODE, 128, G); \
+    else if (d == 64) LGS_RET(MODE, 64, G); \
+    else LGS_RET(MODE, 0, G);           \
+  } while (0)
+    if (side) {  // few sequences and heads: the chunks side by side
+      LGS_RET_D(1, cgrid);
+      lgs::retention_carry_kernel<<<dim3(B, H, (d * dv + 255) / 256), 256, 0, stream>>>(p);
+      LGS_RET_D(2, cgrid);
+    } else {
+      LGS_RET_D(0, cgrid);
     }
-    lgs::retention_chunk_kernel<<<grid, 256, lds, stream>>>(p);
+#undef LGS_RET_D
+#undef LGS_RET
     LGA_LAUNCH_RETURN();
   }
   if (d <= 64) lgs::retention_scan_kernel<16><<<grid, 256, 0, stream>>>(p);
@@ -712,7 +883,10 @@ extern "C" int lgs_latent_attention(const float* qc, const float* proj, long ld,
     if (cache_f32) lgs::latent_attention_kernel<true, NR><<<grid, 256, lds, stream>>>(p, part);        \
     else lgs::latent_attention_kernel<false, NR><<<grid, 256, lds, stream>>>(p, part);                 \
   } while (0)
-  if (r <= 128) LGS_LAT(2);
+  if (r % 8 == 0 && (uintptr_t)cache_c % 16 == 0 && (uintptr_t)qc % 16 == 0) {  // 16-byte loads of the cached rows
+    if (cache_f32) lgs::latent_attention_vec_kernel<true><<<grid, 256, lds, stream>>>(p, part);
+    else lgs::latent_attention_vec_kernel<false><<<grid, 256, lds, stream>>>(p, part);
+  } else if (r <= 128) LGS_LAT(2);
   else if (r <= 256) LGS_LAT(4);
   else LGS_LAT(8);
 #undef LGS_LAT

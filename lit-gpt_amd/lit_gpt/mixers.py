@@ -101,7 +101,7 @@ class Retention(InputReader):
         H, dv = self.H, self.dv
         o = seq_ops.retention(proj, self.off["q"], self.off["k"], self.off["v"], cache.s, self.decay, self.inv_freq,
                               step.seq_start, step.seq_slot, step.seq_pos0, H=H, d=self.d, dv=dv,
-                              rot_dims=self.rot_dims, k_scale=self.k_scale)
+                              rot_dims=self.rot_dims, k_scale=self.k_scale, max_len=step.max_len, pos=step.pos)
         seq_ops.head_gate(o, proj, self.off["g"], H=H, dv=dv, unit_norm=True, eps=self.eps, act=seq_ops.ACT_SILU)
         W = x.shape[1]
         seq_ops.linear(o, self.w_o, M=step.T, N=W, K=H * dv, y=x, lda=H * dv, ldy=W, accumulate=True)

@@ -35,7 +35,7 @@ SIGNATURES = {
     "lgs_embed": [_P, _P, _I, _F, _P, _I, _I, _I, _P],
     "lgs_rmsnorm": [_P, _L, _P, _F, _F, _P, _L, _I, _I, _I, _P],
     "lgs_gather_rows": [_P, _P, _P, _I, _I, _P],
-    "lgs_retention": [_P, _P, _P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P],
+    "lgs_retention": [_P, _P, _P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P, _I, _I, _P, _P],
     "lgs_head_gate": [_P, _P, _L, _I, _I, _I, _I, _F, _I, _P],
     "lgs_latent_prepare": [_P, _L, _I, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P],
     "lgs_latent_attention": [_P, _P, _L, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P],
@@ -141,11 +141,13 @@ def gather_rows(x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
 def retention(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, state: torch.Tensor, decay: torch.Tensor,
               inv_freq: Optional[torch.Tensor], seq_start: torch.Tensor, seq_slot: torch.Tensor,
               seq_pos0: torch.Tensor, *, H: int, d: int, dv: int, rot_dims: int, k_scale: float,
-              chunked: Optional[bool] = None) -> torch.Tensor:
+              chunked: Optional[bool] = None, max_len: int = 0, pos: Optional[torch.Tensor] = None) -> torch.Tensor:
     """proj (T, ld) holds q, k (H * d each) and v (H * dv) at the given column offsets; state (slots, H, d, dv) fp32
     is read (unless a sequence starts at position 0) and left at the step's last token. Returns o (T, H * dv).
     ``chunked`` picks the prompt form (64-token chunks as matrix products) over the token-by-token scan; by default
-    steps that bring 8 or more tokens per sequence on average take it."""
+    steps that bring 8 or more tokens per sequence on average take it. ``max_len`` (the most tokens any sequence
+    brings; 0: unknown) lets the prompt form run its chunks side by side when a sequence has more than one. The
+    prompt form needs ``pos`` (T,) and rotates / scales the q and k columns of ``proj`` in place."""
     T, ld = proj.shape
     B = seq_slot.numel()
     if tuple(state.shape[1:]) != (H, d, dv) or seq_start.numel() != B + 1 or decay.numel() != H:
@@ -155,13 +157,19 @@ def retention(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, state: tor
     out = torch.empty(T, H * dv, dtype=F32, device=proj.device)
     base = _dev(proj, "proj", F32)
     if chunked is None:
-        chunked = T >= 8 * B
+        chunked = T >= 8 * B and pos is not None
+    if chunked and (pos is None or pos.numel() != T):
+        raise ValueError("retention: the prompt form needs the rows' positions")
+    ws, max_chunks = None, 0
+    if chunked and d <= 128 and max_len > 64:
+        max_chunks = (max_len + 63) // 64
+        ws = torch.empty(B * max_chunks * H * d * dv, dtype=F32, device=proj.device)
     _check(load_library().lgs_retention(base + 4 * q_off, base + 4 * k_off, base + 4 * v_off, ld,
                                         _dev(state, "state", F32), _dev(decay, "decay", F32),
                                         _opt(inv_freq, "inv_freq", F32), _dev(seq_start, "seq_start", I32),
                                         _dev(seq_slot, "seq_slot", I32), _dev(seq_pos0, "seq_pos0", I32),
                                         out.data_ptr(), B, H, d, dv, rot_dims, float(k_scale), int(bool(chunked)),
-                                        _stream()))
+                                        _opt(ws, "ws", F32), max_chunks, T, _opt(pos, "pos", I32), _stream()))
     return out
 
 

@@ -339,13 +339,16 @@ def test_retention_far_token_survives():
     ld = 2 * H * d + H * dv
     proj = torch.cat([q.reshape(T, -1), k.reshape(T, -1), v.reshape(T, -1)], 1).contiguous().to(dev)
     dec = torch.tensor(decay, device=dev)
-    for cuts in ([T], [500] + [1] * 20, [64] * 8 + [8], [2] * 260):
+    for cuts, side_by_side in (([T], True), ([T], False), ([500] + [1] * 20, True), ([64] * 8 + [8], False),
+                               ([200, 129, 191], True), ([2] * 260, False)):
         state = torch.full((3, H, d, dv), 7.0, device=dev)  # stale values of an earlier owner of the slot
         outs, at = [], 0
         for n in cuts:
             i32 = lambda *x: torch.tensor(x, dtype=torch.int32, device=dev)  # noqa: E731
             outs.append(seq_ops.retention(proj[at:at + n].contiguous(), 0, H * d, 2 * H * d, state, dec, None,
-                                          i32(0, n), i32(2), i32(at), H=H, d=d, dv=dv, rot_dims=0, k_scale=1.0))
+                                          i32(0, n), i32(2), i32(at), H=H, d=d, dv=dv, rot_dims=0, k_scale=1.0,
+                                          max_len=n if side_by_side else 0,
+                                          pos=torch.arange(at, at + n, dtype=torch.int32, device=dev)))
             at += n
         got = torch.cat(outs).cpu().view(T, H, dv).double()
         assert (got - want).abs().max() < 1e-4 * want.abs().max(), cuts
