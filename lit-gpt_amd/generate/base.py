@@ -272,6 +272,14 @@ def main(prompt: str = "What food do llamas eat?", *, num_samples: int = 1, max_
         raise NotImplementedError("the MI355X path computes in bf16 (bf16-true) or fp32 (32-true)")
     dtype = torch.float32 if precision == "32-true" else torch.bfloat16
     device = torch.device("cuda", torch.cuda.current_device())
+    if synthetic is None and (Path(checkpoint_dir) / "config.json").is_file():
+        from lit_gpt.config import LayeredConfig, load_config
+
+        layered = load_config(checkpoint_dir)
+        if isinstance(layered, LayeredConfig):  # config.json names a registered layered architecture
+            return _main_layered(layered, Path(checkpoint_dir), prompt, num_samples=num_samples,
+                                 max_new_tokens=max_new_tokens, top_k=top_k, temperature=temperature, dtype=dtype,
+                                 device=device, prompt_len=prompt_len, quantize=quantize)
     tokenizer = None
     if synthetic is not None:
         config = Config.from_name(synthetic)
@@ -308,6 +316,45 @@ def main(prompt: str = "What food do llamas eat?", *, num_samples: int = 1, max_
         tokens_generated = y.size(0) - prompt_length
         print(f"Time for inference {i + 1}: {t:.02f} sec total, {tokens_generated / t:.02f} tokens/sec",
               file=sys.stderr)
+    print(f"Memory used: {torch.cuda.max_memory_allocated() / 1e9:.02f} GB", file=sys.stderr)
+
+
+def _main_layered(config, checkpoint_dir: Path, prompt: str, *, num_samples: int, max_new_tokens: int,
+                  top_k: Optional[int], temperature: float, dtype: torch.dtype, device: torch.device, prompt_len: int,
+                  quantize: Optional[str]) -> None:
+    """``main`` for a checkpoint folder whose config.json names a layered architecture (lit_gpt.config.ARCHITECTURES):
+    config.json + model.safetensors, bf16 or fp32 weights, the same generate / sample path. Without tokenizer files
+    the prompt is ``--prompt_len`` synthetic token ids and the output is printed as ids."""
+    from lit_gpt import seq_ops
+    from lit_gpt.config import model_class
+
+    if quantize is not None:
+        raise NotImplementedError("the layered models run bf16 or fp32 weights")
+    seq_ops.build_library()
+    tokenizer = None
+    if (checkpoint_dir / "tokenizer.json").is_file() or (checkpoint_dir / "tokenizer.model").is_file():
+        from lit_gpt.tokenizer import Tokenizer
+
+        tokenizer = Tokenizer(checkpoint_dir)
+        encoded = tokenizer.encode(prompt, device=device).to(torch.int32)
+    else:
+        g = torch.Generator(device="cpu").manual_seed(1234)
+        encoded = torch.randint(0, config.vocab, (prompt_len,), generator=g, dtype=torch.int32).to(device)
+    t0 = time.perf_counter()
+    model = model_class(config).from_checkpoint(checkpoint_dir, device=device, dtype=dtype)
+    print(f"Time to load the model weights: {time.perf_counter() - t0:.02f} seconds.", file=sys.stderr)
+    T = encoded.size(0)
+    model.set_kv_cache(1, T + max_new_tokens)
+    torch.manual_seed(1234)
+    for i in range(num_samples):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        y = generate(model, encoded, T + max_new_tokens, temperature=temperature, top_k=top_k,
+                     eos_id=tokenizer.eos_id if tokenizer is not None else None)
+        torch.cuda.synchronize()
+        t = time.perf_counter() - t0
+        print(tokenizer.decode(y) if tokenizer is not None else y.tolist())
+        print(f"Time for inference {i + 1}: {t:.02f} sec total, {(y.size(0) - T) / t:.02f} tokens/sec", file=sys.stderr)
     print(f"Memory used: {torch.cuda.max_memory_allocated() / 1e9:.02f} GB", file=sys.stderr)
 
 

@@ -507,3 +507,34 @@ def test_checkpoint_folder_round_trip(tmp_path):
     toks = tokens_of(11, cfg["vocab"])
     got = engine_logits(model, [toks], [[11]])[0]
     assert rel_err(got, oracle_logits(cfg, w, toks)).max() < TOL32
+
+
+def test_command_line_serves_a_checkpoint_folder(tmp_path, capsys):
+    """generate/base.py's main on a folder with config.json + model.safetensors of a registered architecture."""
+    import json
+    import struct
+
+    from generate.base import main
+    from lit_gpt.config import LayeredConfig
+    from lit_gpt.layered import LayeredGPT
+
+    cfg = make_cfg(MIXED[:2], vocab=70)
+    w = LayeredGPT.random_weights(LayeredConfig.from_dict(cfg), seed=15)
+    header, blob = {}, b""
+    for name, t in w.items():
+        raw = t.contiguous().view(torch.uint8).numpy().tobytes()
+        header[name] = {"dtype": "BF16", "shape": list(t.shape), "data_offsets": [len(blob), len(blob) + len(raw)]}
+        blob += raw
+    hj = json.dumps(header).encode()
+    (tmp_path / "model.safetensors").write_bytes(struct.pack("<Q", len(hj)) + hj + blob)
+    (tmp_path / "config.json").write_text(json.dumps(cfg))
+    main(checkpoint_dir=tmp_path, max_new_tokens=5, temperature=0.0, top_k=None, prompt_len=7, precision="32-true")
+    ids = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+    assert len(ids) == 12
+    g = torch.Generator(device="cpu").manual_seed(1234)
+    prompt = torch.randint(0, 70, (7,), generator=g, dtype=torch.int32).tolist()
+    assert ids[:7] == prompt
+    lg = oracle_logits(cfg, w, ids[:-1])
+    agree = [ids[i + 1] == int(torch.argmax(lg[i])) for i in range(6, 11)
+             if float(torch.topk(lg[i], 2).values.diff().abs()) > 1e-3]
+    assert agree and all(agree)
