@@ -49,7 +49,7 @@ int lgs_gather_rows(const float* x, const int* rows, float* y, int n_rows, int W
 
 /* retention: rotary (pairs i, i + rot_dims/2; angle = position * inv_freq[i]) on q and k, k * k_scale, then per
  * sequence and head S <- decay S + k v^T, o = S^T q. state [slots][H][d][dv] fp32 is read unless the sequence's
- * first position is 0 and written back at the end of the step. d <= 256. chunked != 0 (and d <= 128) runs the
+ * first position is 0 and written back at the end of the step. d <= 512. chunked != 0 (and d <= 128) runs the
  * prompt form: chunks of 64 tokens as fp32 matrix products, the state carried from chunk to chunk in LDS; with a
  * workspace ws of B * max_chunks * H * d * dv floats (max_chunks = 64-token chunks of the longest sequence) the chunks
  * run side by side when sequences and heads alone would not fill the chip: local sums, a short carry over the

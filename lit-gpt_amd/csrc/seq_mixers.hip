@@ -36,10 +36,10 @@ struct RetArgs {
 // grid (B, H, ceil(dv / 64)): a workgroup owns 64 columns of one head's state; wave w owns rows [w NR, (w + 1) NR)
 template <int NR>
 __global__ void __launch_bounds__(256) retention_scan_kernel(RetArgs p) {
-  __shared__ float qs[256], ks[256];
+  __shared__ float qs[512], ks[512];
   __shared__ float part[4][64];
   const int b = blockIdx.x, h = blockIdx.y, col = blockIdx.z * 64 + (threadIdx.x & 63);
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, tid = threadIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int d = p.d, dv = p.dv, half = p.rot_dims / 2;
   const int t0 = p.seq_start[b], t1 = p.seq_start[b + 1];
   const int pos0 = p.seq_pos0[b];
@@ -54,7 +54,7 @@ __global__ void __launch_bounds__(256) retention_scan_kernel(RetArgs p) {
   }
   for (int t = t0; t < t1; ++t) {
     const float pos = (float)(pos0 + (t - t0));
-    if (tid < d) {
+    for (int tid = threadIdx.x; tid < d; tid += 256) {
       const float* qr = p.q + (size_t)t * p.ld + (size_t)h * d;
       const float* kr = p.k + (size_t)t * p.ld + (size_t)h * d;
       float qo = qr[tid], ko = kr[tid];
@@ -797,7 +797,7 @@ extern "C" int lgs_retention(float* q, float* k, const float* v, long ld, float*
                              float* out, int B, int H, int d, int dv, int rot_dims, float k_scale, int chunked,
                              float* ws, int max_chunks, int T_rows, const int* pos, hipStream_t stream) {
   LGA_CHECK_ARG(q && k && v && state && decay && seq_start && seq_slot && seq_pos0 && out, "lgs_retention: null pointer");
-  LGA_CHECK_ARG(B > 0 && H > 0 && H <= 65535 && d > 0 && d <= 256 && dv > 0, "lgs_retention: head dim must be in [1, 256]");
+  LGA_CHECK_ARG(B > 0 && H > 0 && H <= 65535 && d > 0 && d <= 512 && dv > 0, "lgs_retention: head dim must be in [1, 512]");
   LGA_CHECK_ARG(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= d && (rot_dims == 0 || inv_freq),
                 "lgs_retention: bad rotary dims");
   LGA_CHECK_ARG(!ws || max_chunks > 0, "lgs_retention: a workspace needs the longest sequence's chunk count");
@@ -840,7 +840,8 @@ extern "C" int lgs_retention(float* q, float* k, const float* v, long ld, float*
   }
   if (d <= 64) lgs::retention_scan_kernel<16><<<grid, 256, 0, stream>>>(p);
   else if (d <= 128) lgs::retention_scan_kernel<32><<<grid, 256, 0, stream>>>(p);
-  else lgs::retention_scan_kernel<64><<<grid, 256, 0, stream>>>(p);
+  else if (d <= 256) lgs::retention_scan_kernel<64><<<grid, 256, 0, stream>>>(p);
+  else lgs::retention_scan_kernel<128><<<grid, 256, 0, stream>>>(p);
   LGA_LAUNCH_RETURN();
 }
 
