@@ -35,16 +35,18 @@ int lgs_version(void);
  * ([N][K]), y[z] = y + z stride_y (row stride ldy). M <= 8: streaming GEMV; otherwise 128x128 MFMA tiles (bf16) or
  * 64x64 FMA tiles (fp32). z_start (batch + 1 bounds, device) makes it grouped: batch z owns rows
  * [z_start[z], z_start[z+1]) of a list of at most M rows; list row i reads A row a_rows[i] (or i) and writes Y row i
- * (stride_a and stride_y are then ignored for the rows' place). */
-int lgs_linear(const float* a, long lda, long stride_a, const void* w, int w_f32, long stride_w, float* y, long ldy,
+ * (stride_a and stride_y are then ignored for the rows' place). a_bf16: A is a producer's bf16 copy (MFMA tiles with
+ * bf16 weights only): the same values the fp32 stream would be rounded to, at half the operand traffic. y_bf16: the
+ * result is written as bf16 (it feeds another bf16 product; MFMA tiles, no accumulate). */
+int lgs_linear(const void* a, long lda, long stride_a, const void* w, int w_f32, long stride_w, void* y, long ldy,
                long stride_y, int M, int N, int K, int batch, int accumulate, int act, const int* a_rows,
-               const int* z_start, lgs_stream_t stream);
+               const int* z_start, int a_bf16, int y_bf16, lgs_stream_t stream);
 /* x[t] = table[tokens[t]] * scale */
 int lgs_embed(const int* tokens, const void* table, int w_f32, float scale, float* x, int T, int W, int vocab,
               lgs_stream_t stream);
 /* group g of row r: y = x / sqrt(mean(x^2) + eps) * (offset + weight) (weight NULL: unit RMS), n values per group */
 int lgs_rmsnorm(const float* x, long ldx, const float* weight, float offset, float eps, float* y, long ldy, int rows,
-                int groups, int n, lgs_stream_t stream);
+                int groups, int n, void* y_bf16 /* optional rounded copy, same layout */, lgs_stream_t stream);
 int lgs_gather_rows(const float* x, const int* rows, float* y, int n_rows, int W, lgs_stream_t stream);
 
 /* retention: rotary (pairs i, i + rot_dims/2; angle = position * inv_freq[i]) on q and k, k * k_scale, then per
@@ -61,7 +63,7 @@ int lgs_retention(float* q, float* k, const float* v, long ld, float* state, con
                   int T_rows, const int* pos, lgs_stream_t stream);
 /* in place on o [T][H][dv]: (unit_norm ? o / rms(o) per head : o) * act(g[t * ldg + h * dv + i]) */
 int lgs_head_gate(float* o, const float* g, long ldg, int T, int H, int dv, int unit_norm, float eps, int act,
-                  lgs_stream_t stream);
+                  void* o_bf16 /* optional rounded copy [T][H * dv] */, lgs_stream_t stream);
 /* latent attention, per token: c = rmsnorm(proj[kv_off .. + r]) * norm_w -> cache_c[slot][pos] (bf16, or fp32 with
  * cache_f32); rotary (pairs 2i, 2i + 1) of proj[kv_off + r .. + dr] -> cache_kr[slot][pos] (fp32); the rotated
  * part of every head's query (at q_off + h (d + dr) + d) is rotated in place. */
@@ -84,7 +86,8 @@ int lgs_latent_attention_tiles(const float* qc, const float* proj, long ld, int 
                                int dr, int r, int max_seq, float scale, lgs_stream_t stream);
 
 /* out[t][i] = act(a[t * ld + i]) * b[t * ld + i], i < n */
-int lgs_glu(const float* a, const float* b, long ld, float* out, int T, int n, int act, lgs_stream_t stream);
+int lgs_glu(const float* a, const float* b, long ld, void* out /* fp32, or bf16 with out_bf16 */, int out_bf16, int T,
+            int n, int act, lgs_stream_t stream);
 /* per token: ids / wts [T][top] = the top largest of z[t * ld .. + E] (lowest index first among equals) and the
  * softmax over those. E <= 256. */
 int lgs_moe_route(const float* z, long ld, int T, int E, int top, int* ids, float* wts, lgs_stream_t stream);

@@ -14,10 +14,13 @@
 namespace lgs {
 
 __global__ void __launch_bounds__(256) glu_kernel(const float* __restrict__ a, const float* __restrict__ b, long ld,
-                                                  float* __restrict__ out, int n, int act) {
+                                                  float* __restrict__ out, uint16_t* __restrict__ out16, int n, int act) {
   const size_t t = blockIdx.y;
   const int i = blockIdx.x * 256 + threadIdx.x;
-  if (i < n) out[t * n + i] = act_f(act, a[t * ld + i]) * b[t * ld + i];
+  if (i >= n) return;
+  const float v = act_f(act, a[t * ld + i]) * b[t * ld + i];
+  if (out16) out16[t * n + i] = f2bf(v);  // the operand of a bf16 product: rounded here instead of at its load
+  else out[t * n + i] = v;
 }
 
 // one wave per token; lane holds logits lane + 64 e (E <= 256)
@@ -223,10 +226,11 @@ __global__ void __launch_bounds__(256) token_side_kernel(float* __restrict__ x, 
 
 }  // namespace lgs
 
-extern "C" int lgs_glu(const float* a, const float* b, long ld, float* out, int T, int n, int act,
+extern "C" int lgs_glu(const float* a, const float* b, long ld, void* out, int out_bf16, int T, int n, int act,
                        hipStream_t stream) {
   LGA_CHECK_ARG(a && b && out && T > 0 && T <= 65535 && n > 0, "lgs_glu: bad arguments");
-  lgs::glu_kernel<<<dim3((n + 255) / 256, T), 256, 0, stream>>>(a, b, ld, out, n, act);
+  lgs::glu_kernel<<<dim3((n + 255) / 256, T), 256, 0, stream>>>(a, b, ld, out_bf16 ? nullptr : (float*)out,
+                                                                 out_bf16 ? (uint16_t*)out : nullptr, n, act);
   LGA_LAUNCH_RETURN();
 }
 

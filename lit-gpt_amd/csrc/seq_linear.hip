@@ -26,6 +26,8 @@ struct LinArgs {
   int accumulate, act;
   const int* a_rows;   // row r of the list reads A row a_rows[r] (null: r)
   const int* z_start;  // batch z owns list rows [z_start[z], z_start[z + 1]) (null: rows [0, M) in every batch)
+  const uint16_t* a16;  // MFMA tiles only: A as bf16 (a producer's rounded copy) instead of fp32 `a`
+  uint16_t* y16;        // MFMA tiles only: Y written as bf16 (the operand of a following bf16 product), no accumulate
 };
 
 // ------------------------------------------------------------------------------------------------ GEMV, M <= 8
@@ -113,8 +115,9 @@ constexpr int BM = 128, BN = 128, BK = 64;
 constexpr int TILE_BYTES = BM * BK * 2;
 __device__ __forceinline__ int swz(int row, int chunk) { return row * 128 + 16 * (chunk ^ (row & 7)); }
 
-// VEC: K % 8 == 0 and 16-B aligned rows of A and W (vector loads); otherwise element loads with k guards
-template <bool VEC>
+// VEC: K % 8 == 0 and 16-B aligned rows of A and W (vector loads); otherwise element loads with k guards.
+// A16: A arrives as bf16 (half the operand traffic of the fp32 stream; the same values the fp32 path would round to)
+template <bool VEC, bool A16>
 __global__ void __launch_bounds__(256) lin_mfma_kernel(LinArgs p) {
   __shared__ __attribute__((aligned(16))) unsigned char lds[2 * 2 * TILE_BYTES];  // [buf][A|W]
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -124,12 +127,15 @@ __global__ void __launch_bounds__(256) lin_mfma_kernel(LinArgs p) {
   const int Mz = p.z_start ? p.z_start[z + 1] - r_lo : p.M;
   const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
   if (m0 >= Mz) return;
-  const float* abase = p.a + (size_t)z * p.sa;
+  const float* abase = A16 ? nullptr : p.a + (size_t)z * p.sa;
+  const uint16_t* abase16 = A16 ? p.a16 + (size_t)z * p.sa : nullptr;
   const uint16_t* wbase = (const uint16_t*)p.w + (size_t)z * p.sw;
   const int K = p.K, nk = (K + BK - 1) / BK;
   const int t_row = tid >> 1, t_half = tid & 1;
   const int lr = r_lo + min(m0 + t_row, Mz - 1);  // rows past the end repeat the last one (never stored)
-  const float* arow = abase + (size_t)(p.a_rows ? p.a_rows[lr] : lr) * p.lda;
+  const size_t arow_off = (size_t)(p.a_rows ? p.a_rows[lr] : lr) * p.lda;
+  const float* arow = abase + arow_off;
+  const uint16_t* arow16 = abase16 + arow_off;
   const uint16_t* wrow = wbase + (size_t)min(n0 + t_row, p.N - 1) * K;
 
   uint4 areg[4], wreg[4];
@@ -140,8 +146,12 @@ __global__ void __launch_bounds__(256) lin_mfma_kernel(LinArgs p) {
       for (int c = 0; c < 4; ++c) {
         const int k = k0 + c * 8;
         if (k < K) {
-          const float4 lo = *(const float4*)(arow + k), hi = *(const float4*)(arow + k + 4);
-          areg[c] = make_uint4(pack2(lo.x, lo.y), pack2(lo.z, lo.w), pack2(hi.x, hi.y), pack2(hi.z, hi.w));
+          if (A16) {
+            areg[c] = *(const uint4*)(arow16 + k);
+          } else {
+            const float4 lo = *(const float4*)(arow + k), hi = *(const float4*)(arow + k + 4);
+            areg[c] = make_uint4(pack2(lo.x, lo.y), pack2(lo.z, lo.w), pack2(hi.x, hi.y), pack2(hi.z, hi.w));
+          }
           wreg[c] = *(const uint4*)(wrow + k);
         } else {
           areg[c] = make_uint4(0, 0, 0, 0);
@@ -155,9 +165,14 @@ __global__ void __launch_bounds__(256) lin_mfma_kernel(LinArgs p) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int k = k0 + c * 8 + 2 * e;
-          const float a0 = k < K ? arow[k] : 0.0f, a1 = k + 1 < K ? arow[k + 1] : 0.0f;
           const uint32_t w0 = k < K ? wrow[k] : 0, w1 = k + 1 < K ? wrow[k + 1] : 0;
-          av[e] = pack2(a0, a1);
+          if (A16) {
+            const uint32_t b0 = k < K ? arow16[k] : 0, b1 = k + 1 < K ? arow16[k + 1] : 0;
+            av[e] = b0 | (b1 << 16);
+          } else {
+            const float a0 = k < K ? arow[k] : 0.0f, a1 = k + 1 < K ? arow[k + 1] : 0.0f;
+            av[e] = pack2(a0, a1);
+          }
           wv[e] = w0 | (w1 << 16);
         }
         areg[c] = make_uint4(av[0], av[1], av[2], av[3]);
@@ -207,7 +222,6 @@ __global__ void __launch_bounds__(256) lin_mfma_kernel(LinArgs p) {
     __syncthreads();
   }
 
-  float* ybase = p.y + (size_t)z * p.sy;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int n = n0 + wn * 64 + j * 16 + fr;
@@ -218,9 +232,10 @@ __global__ void __launch_bounds__(256) lin_mfma_kernel(LinArgs p) {
       for (int r = 0; r < 4; ++r) {
         const int m = m0 + wm * 64 + i * 16 + fk * 4 + r;
         if (m >= Mz) continue;
-        float* yp = ybase + (size_t)(r_lo + m) * p.ldy + n;
+        const size_t at = (size_t)z * p.sy + (size_t)(r_lo + m) * p.ldy + n;
         const float v = act_f(p.act, acc[i][j][r]);
-        *yp = p.accumulate ? *yp + v : v;
+        if (p.y16) p.y16[at] = f2bf(v);
+        else p.y[at] = p.accumulate ? p.y[at] + v : v;
       }
   }
 }
@@ -306,7 +321,8 @@ __global__ void __launch_bounds__(256) embed_kernel(const int* __restrict__ tok,
 
 // grid (rows, groups): group g of row r is x[r * ldx + g * n .. + n); weight (may be null) is indexed within a group
 __global__ void __launch_bounds__(256) rmsnorm_kernel(const float* __restrict__ x, long ldx, const float* __restrict__ w,
-                                                      float offset, float eps, float* __restrict__ y, long ldy, int n) {
+                                                      float offset, float eps, float* __restrict__ y, long ldy, int n,
+                                                      uint16_t* __restrict__ y16) {
   __shared__ float red[4];
   const float* xr = x + (size_t)blockIdx.x * ldx + (size_t)blockIdx.y * n;
   float* yr = y + (size_t)blockIdx.x * ldy + (size_t)blockIdx.y * n;
@@ -314,7 +330,12 @@ __global__ void __launch_bounds__(256) rmsnorm_kernel(const float* __restrict__ 
   for (int i = threadIdx.x; i < n; i += 256) ss = fmaf(xr[i], xr[i], ss);
   ss = block_sum_256(ss, red);
   const float rstd = 1.0f / sqrtf(ss / (float)n + eps);
-  for (int i = threadIdx.x; i < n; i += 256) yr[i] = xr[i] * rstd * (w ? offset + w[i] : 1.0f);
+  uint16_t* yb = y16 ? y16 + (size_t)blockIdx.x * ldy + (size_t)blockIdx.y * n : nullptr;
+  for (int i = threadIdx.x; i < n; i += 256) {
+    const float v = xr[i] * rstd * (w ? offset + w[i] : 1.0f);
+    yr[i] = v;
+    if (yb) yb[i] = f2bf(v);  // the rounded copy the matrix cores read
+  }
 }
 
 // y[i] = x[rows[i]] (row gather of the positions whose logits are asked for)
@@ -326,14 +347,21 @@ __global__ void __launch_bounds__(256) gather_rows_kernel(const float* __restric
 
 }  // namespace lgs
 
-extern "C" int lgs_linear(const float* a, long lda, long stride_a, const void* w, int w_f32, long stride_w, float* y,
+extern "C" int lgs_linear(const void* a_any, long lda, long stride_a, const void* w, int w_f32, long stride_w, void* y_any,
                           long ldy, long stride_y, int M, int N, int K, int batch, int accumulate, int act,
-                          const int* a_rows, const int* z_start, hipStream_t stream) {
+                          const int* a_rows, const int* z_start, int a_bf16, int y_bf16, hipStream_t stream) {
+  const float* a = (const float*)a_any;  // (bf16 when a_bf16)
+  float* y = (float*)y_any;              // (bf16 when y_bf16)
   LGA_CHECK_ARG(a && w && y, "lgs_linear: null pointer");
+  LGA_CHECK_ARG(!a_bf16 || (!w_f32 && (M > 8 || z_start || a_rows)),
+                "lgs_linear: a bf16 A operand goes with bf16 weights on the MFMA tiles (more than 8 rows)");
   LGA_CHECK_ARG(M > 0 && N > 0 && K > 0 && batch > 0 && batch <= 65535, "lgs_linear: bad sizes");
   LGA_CHECK_ARG(lda >= K && ldy >= N, "lgs_linear: row strides shorter than the rows");
   LGA_CHECK_ARG(act >= 0 && act <= lgs::kActSigmoid, "lgs_linear: unknown activation");
-  lgs::LinArgs p{a, lda, stride_a, w, stride_w, y, ldy, stride_y, M, N, K, accumulate, act, a_rows, z_start};
+  LGA_CHECK_ARG(!y_bf16 || (!w_f32 && !accumulate && (M > 8 || z_start || a_rows)),
+                "lgs_linear: a bf16 result comes from the MFMA tiles (bf16 weights, more than 8 rows, no accumulate)");
+  lgs::LinArgs p{a, lda, stride_a, w, stride_w, y, ldy, stride_y, M, N, K, accumulate, act, a_rows, z_start,
+                 a_bf16 ? (const uint16_t*)a : nullptr, y_bf16 ? (uint16_t*)y : nullptr};
   if (M <= 8 && !z_start && !a_rows) {
     const int R = N >= 16384 ? 4 : (N >= 4096 ? 2 : 1);
     const dim3 grid((N + 4 * R - 1) / (4 * R), batch);
@@ -364,10 +392,16 @@ extern "C" int lgs_linear(const float* a, long lda, long stride_a, const void* w
   }
   const dim3 grid((N + lgs::BN - 1) / lgs::BN, (M + lgs::BM - 1) / lgs::BM, batch);
   LGA_CHECK_ARG(grid.y <= 65535, "lgs_linear: too many rows");
-  const bool vec = K % 8 == 0 && lda % 4 == 0 && stride_a % 4 == 0 && stride_w % 8 == 0 && (uintptr_t)a % 16 == 0 &&
+  const int am = a_bf16 ? 8 : 4;  // elements per 16 bytes of A
+  const bool vec = K % 8 == 0 && lda % am == 0 && stride_a % am == 0 && stride_w % 8 == 0 && (uintptr_t)a % 16 == 0 &&
                    (uintptr_t)w % 16 == 0;
-  if (vec) lgs::lin_mfma_kernel<true><<<grid, 256, 0, stream>>>(p);
-  else lgs::lin_mfma_kernel<false><<<grid, 256, 0, stream>>>(p);
+  if (a_bf16) {
+    if (vec) lgs::lin_mfma_kernel<true, true><<<grid, 256, 0, stream>>>(p);
+    else lgs::lin_mfma_kernel<false, true><<<grid, 256, 0, stream>>>(p);
+  } else {
+    if (vec) lgs::lin_mfma_kernel<true, false><<<grid, 256, 0, stream>>>(p);
+    else lgs::lin_mfma_kernel<false, false><<<grid, 256, 0, stream>>>(p);
+  }
   LGA_LAUNCH_RETURN();
 }
 
@@ -380,9 +414,10 @@ extern "C" int lgs_embed(const int* tokens, const void* table, int w_f32, float 
 }
 
 extern "C" int lgs_rmsnorm(const float* x, long ldx, const float* weight, float offset, float eps, float* y, long ldy,
-                           int rows, int groups, int n, hipStream_t stream) {
+                           int rows, int groups, int n, void* y_bf16, hipStream_t stream) {
   LGA_CHECK_ARG(x && y && rows > 0 && groups > 0 && groups <= 65535 && n > 0, "lgs_rmsnorm: bad arguments");
-  lgs::rmsnorm_kernel<<<dim3(rows, groups), 256, 0, stream>>>(x, ldx, weight, offset, eps, y, ldy, n);
+  lgs::rmsnorm_kernel<<<dim3(rows, groups), 256, 0, stream>>>(x, ldx, weight, offset, eps, y, ldy, n,
+                                                              (uint16_t*)y_bf16);
   LGA_LAUNCH_RETURN();
 }
 

@@ -300,8 +300,10 @@ static size_t retention_chunk_lds(int d) {
 }
 
 // grid (T, H): o[t][h][:] <- (unit ? o / rms(o) : o) * act(g[t * ldg + h * dv + :])
+// (o16: optional rounded copy, the operand of the out-projection's bf16 MFMA tiles)
 __global__ void __launch_bounds__(256) head_gate_kernel(float* __restrict__ o, const float* __restrict__ g, long ldg,
-                                                        int H, int dv, int unit, float eps, int act) {
+                                                        int H, int dv, int unit, float eps, int act,
+                                                        uint16_t* __restrict__ o16) {
   __shared__ float red[4];
   const int t = blockIdx.x, h = blockIdx.y;
   float* orow = o + ((size_t)t * H + h) * dv;
@@ -313,7 +315,11 @@ __global__ void __launch_bounds__(256) head_gate_kernel(float* __restrict__ o, c
     ss = block_sum_256(ss, red);
     rstd = 1.0f / sqrtf(ss / (float)dv + eps);
   }
-  for (int i = threadIdx.x; i < dv; i += 256) orow[i] = orow[i] * rstd * act_f(act, grow[i]);
+  for (int i = threadIdx.x; i < dv; i += 256) {
+    const float v = orow[i] * rstd * act_f(act, grow[i]);
+    orow[i] = v;
+    if (o16) o16[((size_t)t * H + h) * dv + i] = f2bf(v);
+  }
 }
 
 // ------------------------------------------------------------------------------------------------ latent attention
@@ -846,9 +852,9 @@ extern "C" int lgs_retention(float* q, float* k, const float* v, long ld, float*
 }
 
 extern "C" int lgs_head_gate(float* o, const float* g, long ldg, int T, int H, int dv, int unit_norm, float eps,
-                             int act, hipStream_t stream) {
+                             int act, void* o_bf16, hipStream_t stream) {
   LGA_CHECK_ARG(o && g && T > 0 && H > 0 && H <= 65535 && dv > 0, "lgs_head_gate: bad arguments");
-  lgs::head_gate_kernel<<<dim3(T, H), 256, 0, stream>>>(o, g, ldg, H, dv, unit_norm, eps, act);
+  lgs::head_gate_kernel<<<dim3(T, H), 256, 0, stream>>>(o, g, ldg, H, dv, unit_norm, eps, act, (uint16_t*)o_bf16);
   LGA_LAUNCH_RETURN();
 }
 

@@ -65,13 +65,16 @@ class LayeredBlock(nn.Module):
 
     def forward(self, x: torch.Tensor, step: StepBatch, cache: nn.Module) -> None:
         """x (T, width) fp32, updated in place."""
-        h = self.norm1(x)
+        # more than 8 rows run MFMA tiles: with bf16 weights the norm also leaves its output rounded to bf16, which
+        # the tiles read at half the traffic (the values they would round the fp32 stream to)
+        tiles16 = step.T > 8 and self.w_in.dtype == torch.bfloat16
+        h, h16 = self.norm1(x, bf16_copy=True) if tiles16 else (self.norm1(x), None)
         n_in, W = self.w_in.shape
         proj = torch.empty(step.T, n_in, dtype=torch.float32, device=x.device)
-        seq_ops.linear(h, self.w_in, M=step.T, N=n_in, K=W, y=proj, lda=W, ldy=n_in)
+        seq_ops.linear(h16 if tiles16 else h, self.w_in, M=step.T, N=n_in, K=W, y=proj, lda=W, ldy=n_in)
         self.mixer(proj, step, cache, x)
         if self.mlp is not None:
-            self.mlp(proj, h, x)
+            self.mlp(proj, h, x, h16=h16)
         if self.side is not None:
             self.side(x, step.tokens)
 

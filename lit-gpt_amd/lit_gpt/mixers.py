@@ -61,6 +61,12 @@ def _f32(t: torch.Tensor, device) -> torch.Tensor:
     return t.to(device=device, dtype=torch.float32).contiguous()
 
 
+def _tiles16(rows: int, weight: torch.Tensor) -> bool:
+    """Whether a product of ``rows`` rows with ``weight`` runs bf16 MFMA tiles (more than 8 rows, bf16 weights): its
+    producer then hands over the operand already rounded to bf16, at half the traffic."""
+    return rows > 8 and weight.dtype == torch.bfloat16
+
+
 class InputReader(nn.Module):
     """A module that reads columns of the layer's shared input projection."""
 
@@ -102,7 +108,8 @@ class Retention(InputReader):
         o = seq_ops.retention(proj, self.off["q"], self.off["k"], self.off["v"], cache.s, self.decay, self.inv_freq,
                               step.seq_start, step.seq_slot, step.seq_pos0, H=H, d=self.d, dv=dv,
                               rot_dims=self.rot_dims, k_scale=self.k_scale, max_len=step.max_len, pos=step.pos)
-        seq_ops.head_gate(o, proj, self.off["g"], H=H, dv=dv, unit_norm=True, eps=self.eps, act=seq_ops.ACT_SILU)
+        o = seq_ops.head_gate(o, proj, self.off["g"], H=H, dv=dv, unit_norm=True, eps=self.eps, act=seq_ops.ACT_SILU,
+                              bf16_copy=_tiles16(step.T, self.w_o))
         W = x.shape[1]
         seq_ops.linear(o, self.w_o, M=step.T, N=W, K=H * dv, y=x, lda=H * dv, ldy=W, accumulate=True)
 
@@ -158,8 +165,8 @@ class LatentAttention(InputReader):
         att = torch.empty(T, H * dv, dtype=torch.float32, device=proj.device)
         seq_ops.linear(lat, self.w_uv, M=T, N=dv, K=r, y=att, lda=H * r, ldy=H * dv, batch=H, stride_a=r,
                        stride_w=dv * r, stride_y=dv)
-        seq_ops.head_gate(att, proj, self.off["g"], H=H, dv=dv, unit_norm=False, eps=self.eps,
-                          act=seq_ops.ACT_SIGMOID)
+        att = seq_ops.head_gate(att, proj, self.off["g"], H=H, dv=dv, unit_norm=False, eps=self.eps,
+                                act=seq_ops.ACT_SIGMOID, bf16_copy=_tiles16(T, self.w_o))
         W = x.shape[1]
         seq_ops.linear(att, self.w_o, M=T, N=W, K=H * dv, y=x, lda=H * dv, ldy=W, accumulate=True)
 
@@ -180,8 +187,11 @@ class GatedFeedForward(InputReader):
     def in_parts(self):
         return self._in
 
-    def forward(self, proj: torch.Tensor, h: torch.Tensor, x: torch.Tensor) -> None:
-        a = seq_ops.glu(proj, self.off["gate"], self.off["up"], self.ff, self.act)
+    def forward(self, proj: torch.Tensor, h: torch.Tensor, x: torch.Tensor, h16=None) -> None:
+        # (h: the norm output, fp32 or its bf16 copy; for MFMA tiles with bf16 weights the gated product is rounded
+        # where it is made)
+        a = seq_ops.glu(proj, self.off["gate"], self.off["up"], self.ff, self.act,
+                        bf16=_tiles16(proj.shape[0], self.w_down))
         W = x.shape[1]
         seq_ops.linear(a, self.w_down, M=a.shape[0], N=W, K=self.ff, y=x, lda=self.ff, ldy=W, accumulate=True)
 
@@ -213,7 +223,9 @@ class SparseFeedForward(InputReader):
     def in_parts(self):
         return self._in
 
-    def forward(self, proj: torch.Tensor, h: torch.Tensor, x: torch.Tensor) -> None:
+    def forward(self, proj: torch.Tensor, h: torch.Tensor, x: torch.Tensor,
+                h16: Optional[torch.Tensor] = None) -> None:
+        """h: the norm output (fp32); h16: its bf16 copy when the layer made one (the grouped products read it)."""
         T, W = h.shape
         E, top, F = self.E, self.top, self.ff
         ids, wts = seq_ops.moe_route(proj, self.off["router"], E, top)
@@ -223,9 +235,10 @@ class SparseFeedForward(InputReader):
             return
         pairs = T * top
         z_start, tok_of, where = seq_ops.moe_sort(ids, E)
-        a = torch.empty(pairs, F, dtype=torch.float32, device=h.device)
-        seq_ops.linear(h, self.w_up, M=pairs, N=F, K=W, y=a, lda=W, ldy=F, batch=E, stride_w=F * W, act=self.act,
-                       a_rows=tok_of, z_start=z_start)
+        a = torch.empty(pairs, F, dtype=torch.bfloat16 if self.w_down.dtype == torch.bfloat16 else torch.float32,
+                        device=h.device)
+        seq_ops.linear(h if h16 is None else h16, self.w_up, M=pairs, N=F, K=W, y=a, lda=W, ldy=F, batch=E,
+                       stride_w=F * W, act=self.act, a_rows=tok_of, z_start=z_start)
         y = torch.empty(pairs, W, dtype=torch.float32, device=h.device)
         seq_ops.linear(a, self.w_down, M=pairs, N=W, K=F, y=y, lda=F, ldy=W, batch=E, stride_w=W * F, z_start=z_start)
         seq_ops.moe_combine(y, where, wts, x)

@@ -40,9 +40,10 @@ class StreamRMSNorm(nn.Module):
         self.register_buffer("weight", torch.zeros(size) if offset else torch.ones(size))
         self.eps, self.offset = eps, offset
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, bf16_copy: bool = False):
+        """``bf16_copy``: (y, y rounded to bf16) — the second is what a bf16 MFMA product reads."""
         from lit_gpt import seq_ops
 
         if not x.is_cuda:
             _gpu_only("StreamRMSNorm")
-        return seq_ops.rmsnorm(x, self.weight, offset=self.offset, eps=self.eps)
+        return seq_ops.rmsnorm(x, self.weight, offset=self.offset, eps=self.eps, bf16_copy=bf16_copy)

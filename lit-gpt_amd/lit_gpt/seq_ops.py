@@ -31,16 +31,16 @@ _P, _I, _L, _F = ctypes.c_void_p, ctypes.c_int, ctypes.c_long, ctypes.c_float
 SIGNATURES = {
     "lgs_version": [],
     "lgs_last_error_string": [],
-    "lgs_linear": [_P, _L, _L, _P, _I, _L, _P, _L, _L, _I, _I, _I, _I, _I, _I, _P, _P, _P],
+    "lgs_linear": [_P, _L, _L, _P, _I, _L, _P, _L, _L, _I, _I, _I, _I, _I, _I, _P, _P, _I, _I, _P],
     "lgs_embed": [_P, _P, _I, _F, _P, _I, _I, _I, _P],
-    "lgs_rmsnorm": [_P, _L, _P, _F, _F, _P, _L, _I, _I, _I, _P],
+    "lgs_rmsnorm": [_P, _L, _P, _F, _F, _P, _L, _I, _I, _I, _P, _P],
     "lgs_gather_rows": [_P, _P, _P, _I, _I, _P],
     "lgs_retention": [_P, _P, _P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P, _I, _I, _P, _P],
-    "lgs_head_gate": [_P, _P, _L, _I, _I, _I, _I, _F, _I, _P],
+    "lgs_head_gate": [_P, _P, _L, _I, _I, _I, _I, _F, _I, _P, _P],
     "lgs_latent_prepare": [_P, _L, _I, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P],
     "lgs_latent_attention": [_P, _P, _L, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P],
     "lgs_latent_attention_tiles": [_P, _P, _L, _I, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P],
-    "lgs_glu": [_P, _P, _L, _P, _I, _I, _I, _P],
+    "lgs_glu": [_P, _P, _L, _P, _I, _I, _I, _I, _P],
     "lgs_moe_route": [_P, _L, _I, _I, _I, _P, _P, _P],
     "lgs_moe_up": [_P, _L, _P, _I, _P, _P, _I, _I, _I, _I, _I, _P],
     "lgs_moe_down": [_P, _P, _I, _P, _P, _P, _L, _I, _I, _I, _I, _P],
@@ -98,16 +98,19 @@ def linear(a: torch.Tensor, w: torch.Tensor, *, M: int, N: int, K: int, y: torch
            z_start: Optional[torch.Tensor] = None) -> torch.Tensor:
     """y[z] (+)= act(a[z] w[z]^T) over ``batch`` strided operands; offsets and strides count elements. With
     ``z_start`` (batch + 1 int32 row bounds) batch z owns that range of a row list of at most M rows, whose A rows
-    are ``a_rows`` (or the list places themselves) and whose Y rows are the list places."""
-    ap = _dev(a, "a", F32) + 4 * a_off
-    yp = _dev(y, "y", F32) + 4 * y_off
+    are ``a_rows`` (or the list places themselves) and whose Y rows are the list places. ``a`` may be a producer's
+    bf16 copy (``rmsnorm(bf16_copy=True)``, ``glu(bf16=True)``) for the MFMA tiles with bf16 weights."""
+    a16 = a.dtype == torch.bfloat16
+    ap = _dev(a, "a", torch.bfloat16 if a16 else F32) + (2 if a16 else 4) * a_off
+    y16 = y.dtype == torch.bfloat16  # the result feeds another bf16 product
+    yp = _dev(y, "y", torch.bfloat16 if y16 else F32) + (2 if y16 else 4) * y_off
     need_a = a_off + (batch - 1) * stride_a + (0 if a_rows is not None else (M - 1) * lda) + K
     need_y = y_off + (batch - 1) * stride_y * (0 if z_start is not None else 1) + (M - 1) * ldy + N
     if a.numel() < need_a or y.numel() < need_y or w.numel() < (batch - 1) * stride_w + N * K:
         raise ValueError("linear: an operand is smaller than the sizes and strides say")
     _check(load_library().lgs_linear(ap, lda, stride_a, _dev(w, "w"), _wf32(w, "w"), stride_w, yp, ldy, stride_y,
                                      M, N, K, batch, int(accumulate), act, _opt(a_rows, "a_rows", I32),
-                                     _opt(z_start, "z_start", I32), _stream()))
+                                     _opt(z_start, "z_start", I32), int(a16), int(y16), _stream()))
     return y
 
 
@@ -120,15 +123,18 @@ def embed(tokens: torch.Tensor, table: torch.Tensor, scale: float) -> torch.Tens
 
 
 def rmsnorm(x: torch.Tensor, weight: Optional[torch.Tensor], *, offset: float, eps: float,
-            out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Rows of a contiguous (rows, n) tensor: x / sqrt(mean(x^2) + eps) * (offset + weight) (no weight: unit RMS)."""
+            out: Optional[torch.Tensor] = None, bf16_copy: bool = False):
+    """Rows of a contiguous (rows, n) tensor: x / sqrt(mean(x^2) + eps) * (offset + weight) (no weight: unit RMS).
+    ``bf16_copy``: also returns the result rounded to bf16 (the operand of the bf16 MFMA products): (y, y_bf16)."""
     rows, n = x.shape
     y = out if out is not None else torch.empty_like(x)
+    yb = torch.empty(rows, n, dtype=torch.bfloat16, device=x.device) if bf16_copy else None
     if weight is not None and weight.numel() != n:
         raise ValueError("rmsnorm: weight size")
     _check(load_library().lgs_rmsnorm(_dev(x, "x", F32), n, _opt(weight, "weight", F32), float(offset), float(eps),
-                                      _dev(y, "y", F32), n, rows, 1, n, _stream()))
-    return y
+                                      _dev(y, "y", F32), n, rows, 1, n, _opt(yb, "y_bf16", torch.bfloat16),
+                                      _stream()))
+    return (y, yb) if bf16_copy else y
 
 
 def gather_rows(x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
@@ -174,14 +180,17 @@ def retention(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, state: tor
 
 
 def head_gate(o: torch.Tensor, proj: torch.Tensor, g_off: int, *, H: int, dv: int, unit_norm: bool, eps: float,
-              act: int) -> torch.Tensor:
-    """In place on o (T, H * dv): per head optional unit RMS, then times act(gate), the gate at proj[:, g_off:]."""
+              act: int, bf16_copy: bool = False) -> torch.Tensor:
+    """In place on o (T, H * dv): per head optional unit RMS, then times act(gate), the gate at proj[:, g_off:].
+    Returns o, or with ``bf16_copy`` its rounding to bf16 (the operand of a bf16 MFMA product)."""
     T, ld = proj.shape
     if o.shape != (T, H * dv) or g_off + H * dv > ld:
         raise ValueError("head_gate: shapes")
+    o16 = torch.empty(T, H * dv, dtype=torch.bfloat16, device=o.device) if bf16_copy else None
     _check(load_library().lgs_head_gate(_dev(o, "o", F32), _dev(proj, "proj", F32) + 4 * g_off, ld, T, H, dv,
-                                        int(unit_norm), float(eps), act, _stream()))
-    return o
+                                        int(unit_norm), float(eps), act, _opt(o16, "o_bf16", torch.bfloat16),
+                                        _stream()))
+    return o16 if bf16_copy else o
 
 
 def latent_prepare(proj: torch.Tensor, q_off: int, kv_off: int, cache_c: torch.Tensor, cache_kr: torch.Tensor,
@@ -242,13 +251,15 @@ def latent_attention_tiles(qc: torch.Tensor, proj: torch.Tensor, q_off: int, cac
     return out
 
 
-def glu(proj: torch.Tensor, a_off: int, b_off: int, n: int, act: int) -> torch.Tensor:
+def glu(proj: torch.Tensor, a_off: int, b_off: int, n: int, act: int, bf16: bool = False) -> torch.Tensor:
+    """act(proj[:, a_off:a_off + n]) * proj[:, b_off:b_off + n]; ``bf16``: rounded to bf16 (a bf16 product's operand)."""
     T, ld = proj.shape
     if max(a_off, b_off) + n > ld:
         raise ValueError("glu: columns outside the row")
-    out = torch.empty(T, n, dtype=F32, device=proj.device)
+    out = torch.empty(T, n, dtype=torch.bfloat16 if bf16 else F32, device=proj.device)
     base = _dev(proj, "proj", F32)
-    _check(load_library().lgs_glu(base + 4 * a_off, base + 4 * b_off, ld, out.data_ptr(), T, n, act, _stream()))
+    _check(load_library().lgs_glu(base + 4 * a_off, base + 4 * b_off, ld, out.data_ptr(), int(bf16), T, n, act,
+                                  _stream()))
     return out
 
 

@@ -146,7 +146,7 @@ def test_library_exports_every_header_symbol():
         subprocess.run(["make", "-C", str(REPO / "lit-gpt_amd" / "csrc"), "-j8", "seq"], check=True)
     lib = seq_ops.load_library()
     assert lib.lgs_version() >= 1
-    rc = lib.lgs_linear(None, 1, 0, None, 0, 0, None, 1, 0, 1, 1, 1, 1, 0, 0, None, None, None)
+    rc = lib.lgs_linear(None, 1, 0, None, 0, 0, None, 1, 0, 1, 1, 1, 1, 0, 0, None, None, 0, 0, None)
     assert rc != 0 and b"null" in lib.lgs_last_error_string()
     with pytest.raises(RuntimeError, match="GPU tensor"):
         seq_ops.rmsnorm(torch.zeros(2, 8), torch.ones(8), offset=0.0, eps=1e-5)
