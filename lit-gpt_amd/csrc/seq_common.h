@@ -3,7 +3,7 @@
 //
 // Conventions: activations are fp32 in memory in both precisions. A weight matrix is [out][in], either bf16 (raw
 // uint16; the activation operand of a product is then rounded to bf16 and the sum is fp32: the matrix-core
-// contract) or fp32 (everything fp32, plain FMA). Norm weights, decays, sinks and rotary frequencies are fp32.
+// convention) or fp32 (everything fp32, plain FMA). Norm weights, decays, sinks and rotary frequencies are fp32.
 // A step is a packed batch: the tokens of all its sequences lie row after row; per token an int32 cache slot and
 // position, per sequence its first row, slot and first position. Nothing is allocated or synchronised here, every
 // launch goes to the caller's stream, so a step can be captured into a HIP graph.
