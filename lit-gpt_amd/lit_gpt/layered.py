@@ -226,7 +226,7 @@ class LayeredGPT(nn.Module):
 
     def forward(self, idx: torch.Tensor, input_pos: Optional[torch.Tensor] = None, *,
                 last_token_only: bool = False) -> torch.Tensor:
-        """``GPT.forward``'s contract for one sequence in slot 0: (1, T) ids at positions ``input_pos`` (consecutive;
+        """``GPT.forward``'s calling convention for one sequence in slot 0: (1, T) ids at positions ``input_pos`` (consecutive;
         default 0..T-1, which starts the sequence anew) -> (1, T, vocab) fp32 logits, or (1, 1, vocab)."""
         B, T = idx.shape
         if B != 1:

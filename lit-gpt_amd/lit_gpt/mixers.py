@@ -78,7 +78,8 @@ class InputReader(nn.Module):
 
 
 class Retention(InputReader):
-    """Decayed linear attention without softmax or denominator: per head S_t = decay S_{t-1} + k_t v_t^T,
+    """A per-head outer-product memory with a constant decay, read by the query (linear attention, scores neither
+    normalised nor soft-maxed): per head S_t = decay S_{t-1} + k_t v_t^T,
     o_t = S_t^T q_t, rotary positions (pairs i, i + dims/2) on q and k, k scaled by ``k_scale``; each head's output is
     divided by its root mean square, gated with silu(W_g h) and projected."""
 
@@ -117,7 +118,7 @@ class Retention(InputReader):
 class LatentAttention(InputReader):
     """Causal softmax attention whose keys and values are expanded from a cached low-rank latent c (RMS-normed) and
     one rotated key part shared by all heads (interleaved rotary pairs 2i, 2i + 1). The score of head h is
-    (q_h . W_uk,h c + q_rot,h . k_rot) * scale; the denominator also holds exp(sink_h). The kernels never expand
+    (q_h . W_uk,h c + q_rot,h . k_rot) * scale; a learned per-head sink scalar adds its exponential to the softmax normaliser. The kernels never expand
     keys or values: the query is mapped through W_uk,h first (one product per head), attention runs over the cached
     rows [c | k_rot] for all heads alike, and W_uv,h maps the weighted latent back. Output gate sigmoid(W_g h)."""
 
@@ -197,8 +198,8 @@ class GatedFeedForward(InputReader):
 
 
 class SparseFeedForward(InputReader):
-    """Mixture of experts: fp32 router logits, the ``top`` largest chosen, weights = softmax over the chosen logits
-    only, expert = W_down act(W_up h) without biases (``act`` defaults to the square of relu).
+    """Mixture of experts: fp32 router logits, the ``top`` largest selected, weights = softmax restricted to the selected
+    logits, expert = W_down act(W_up h) without biases (``act`` defaults to the square of relu).
 
     Few (token, choice) pairs (decode) stream only the chosen experts' rows through two GEMV launches. A prompt
     sorts its pairs by expert on the device and runs two grouped products over the expert ranges, then sums each
