@@ -72,7 +72,7 @@ int lgs_latent_prepare(float* proj, long ld, int q_off, int kv_off, void* cache_
                        int d, int dr, int r, int rot_dims, int max_seq, float eps, lgs_stream_t stream);
 /* out[t][h] = sum_j p_j c_j over cached rows j <= pos[t] of slot[t], p = softmax over
  * (qc[t][h] . c_j + q_rot[t][h] . kr_j) * scale with exp(sink[h]) added to the denominator (sink NULL: none).
- * r <= 512, dr <= 128. splits > 1 spreads every (token, head)'s keys over that many workgroups (decode: few rows,
+ * r <= 1024, dr <= 128. splits > 1 spreads every (token, head)'s keys over that many workgroups (decode: few rows,
  * long contexts) and merges them in a second launch; part: T * H * splits * (r + 2) floats of workspace. */
 int lgs_latent_attention(const float* qc, const float* proj, long ld, int q_off, const void* cache_c, int cache_f32,
                          const float* cache_kr, const float* sink, const int* slot, const int* pos, float* out, int T,

@@ -878,8 +878,8 @@ extern "C" int lgs_latent_attention(const float* qc, const float* proj, long ld,
                                     const int* pos, float* out, int T, int H, int d, int dr, int r, int max_seq,
                                     float scale, int splits, float* part, hipStream_t stream) {
   LGA_CHECK_ARG(qc && proj && cache_c && cache_kr && slot && pos && out, "lgs_latent_attention: null pointer");
-  LGA_CHECK_ARG(T > 0 && H > 0 && H <= 65535 && r > 0 && r <= 512 && dr >= 0 && dr <= 128 && max_seq > 0,
-                "lgs_latent_attention: latent rank must be <= 512 and the rotated part <= 128");
+  LGA_CHECK_ARG(T > 0 && H > 0 && H <= 65535 && r > 0 && r <= 1024 && dr >= 0 && dr <= 128 && max_seq > 0,
+                "lgs_latent_attention: latent rank must be <= 1024 and the rotated part <= 128");
   LGA_CHECK_ARG(splits >= 1 && splits <= 256 && (splits == 1 || part),
                 "lgs_latent_attention: splits in [1, 256], with a workspace of T * H * splits * (r + 2) floats");
   lgs::LatAttArgs p{qc, proj, ld, q_off, cache_c, cache_kr, sink, slot, pos, out, H, d, dr, r, max_seq, scale};
@@ -890,12 +890,13 @@ extern "C" int lgs_latent_attention(const float* qc, const float* proj, long ld,
     if (cache_f32) lgs::latent_attention_kernel<true, NR><<<grid, 256, lds, stream>>>(p, part);        \
     else lgs::latent_attention_kernel<false, NR><<<grid, 256, lds, stream>>>(p, part);                 \
   } while (0)
-  if (r % 8 == 0 && (uintptr_t)cache_c % 16 == 0 && (uintptr_t)qc % 16 == 0) {  // 16-byte loads of the cached rows
+  if (r % 8 == 0 && r <= 512 && (uintptr_t)cache_c % 16 == 0 && (uintptr_t)qc % 16 == 0) {  // 16-byte row loads
     if (cache_f32) lgs::latent_attention_vec_kernel<true><<<grid, 256, lds, stream>>>(p, part);
     else lgs::latent_attention_vec_kernel<false><<<grid, 256, lds, stream>>>(p, part);
   } else if (r <= 128) LGS_LAT(2);
   else if (r <= 256) LGS_LAT(4);
-  else LGS_LAT(8);
+  else if (r <= 512) LGS_LAT(8);
+  else LGS_LAT(16);
 #undef LGS_LAT
   if (splits > 1) lgs::latent_combine_kernel<<<dim3(T, H), 256, 0, stream>>>(part, sink, out, H, r, splits);
   LGA_LAUNCH_RETURN();

@@ -156,7 +156,7 @@ class LatentAttention(InputReader):
         qc = torch.empty(T, H * r, dtype=torch.float32, device=proj.device)
         seq_ops.linear(proj, self.w_ukT, M=T, N=r, K=d, y=qc, a_off=q_off, lda=ld, ldy=H * r, batch=H,
                        stride_a=d + dr, stride_w=r * d, stride_y=r)
-        if r % 64 == 0 and T >= 8 * step.B:  # a prompt: 16-token tiles on the matrix cores
+        if r % 64 == 0 and r <= 512 and T >= 8 * step.B:  # a prompt: 16-token tiles on the matrix cores
             lat = seq_ops.latent_attention_tiles(qc, proj, q_off, cache.c, cache.kr, self.sink, step.seq_start,
                                                  step.seq_slot, step.seq_pos0, step.max_len or T, H=H, d=d, dr=dr,
                                                  r=r, scale=self.scale)

@@ -120,6 +120,7 @@ TOL32, TOL16 = 2e-4, 6e-2
     ([(lat(heads=3, dim=16, rot_dim=72, vdim=8, kv_rank=136), None)], 0),
     ([(lat(heads=2, dim=8, rot_dim=6, vdim=8, kv_rank=64), None)], 0),
     ([(lat(heads=2, dim=8, rot_dim=72, vdim=8, kv_rank=128), None)], 0),
+    ([(lat(heads=1, dim=8, rot_dim=4, vdim=8, kv_rank=640), None)], 0),
     ([(ret(heads=1, dim=272, vdim=16, rot_dims=20), None)], 0),
     ([(lat(heads=2, dim=8, rot_dim=16, vdim=24, kv_rank=192), dense())], 0),
     ([(ret(), dense())], 0),
