@@ -53,18 +53,42 @@ _RESTYPES = {"lgs_last_error_string": ctypes.c_char_p}
 _lib: Optional[ctypes.CDLL] = None
 
 
+def _user_lib_path() -> Path:
+    """Where the library goes when the checkout's own folders cannot be written to."""
+    home = Path(os.environ.get("XDG_CACHE_HOME") or Path(os.environ.get("HOME") or "/tmp") / ".cache")
+    return home / "litgpt_amd" / "liblitgpt_seq.so"
+
+
 def build_library() -> Path:
-    """Compile the library in-tree (``make seq``: hipcc --offload-arch=gfx950) unless it is there already."""
-    if not LIB_PATH.is_file():
-        jobs = str(min(16, os.cpu_count() or 8))
-        subprocess.run(["make", "-C", str(CSRC), f"-j{jobs}", "seq"], check=True, stdout=subprocess.DEVNULL)
+    """Compile the library (``make seq``: hipcc --offload-arch=gfx950) unless it is there already: in-tree, or, when
+    the tree's folders are not writable for this user, under the user's cache folder."""
+    global LIB_PATH
+    if LIB_PATH.is_file():
+        return LIB_PATH
+    jobs = str(min(16, os.cpu_count() or 8))
+    try:
+        subprocess.run(["make", "-C", str(CSRC), f"-j{jobs}", "seq"], check=True, stdout=subprocess.DEVNULL,
+                       stderr=subprocess.PIPE)
+    except (subprocess.CalledProcessError, OSError) as first:
+        alt = _user_lib_path()
+        if not alt.is_file():
+            try:
+                alt.parent.mkdir(parents=True, exist_ok=True)
+                subprocess.run(["make", "-C", str(CSRC), f"-j{jobs}", "seq", f"SEQ_BUILD={alt.parent / 'build'}",
+                                f"SEQ_OUT={alt}"], check=True, stdout=subprocess.DEVNULL, stderr=subprocess.PIPE)
+            except (subprocess.CalledProcessError, OSError) as second:
+                err = getattr(second, "stderr", b"") or getattr(first, "stderr", b"") or b""
+                raise NativeLibraryError("building liblitgpt_seq.so failed:\n" + err.decode(errors="replace")[-2000:])
+        LIB_PATH = alt
     return LIB_PATH
 
 
 def load_library() -> ctypes.CDLL:
-    global _lib
+    global _lib, LIB_PATH
     if _lib is not None:
         return _lib
+    if not LIB_PATH.is_file() and _user_lib_path().is_file():
+        LIB_PATH = _user_lib_path()
     if not LIB_PATH.is_file():
         raise NativeLibraryError(f"HIP library not found at {LIB_PATH}. Build it with `make -C lit-gpt_amd/csrc seq` "
                                  "(hipcc --offload-arch=gfx950). There is no CPU fallback.")
