@@ -486,6 +486,33 @@ def test_greedy_generation_through_entry_point_and_scheduler():
     assert checked > 2 * new
 
 
+def test_captured_decode_steps_equal_eager_steps():
+    """The one-token steps as replays of one HIP graph: every replay must give the eager step's token and leave the
+    caches and states as the eager step would, also after other eager work and a second capture in between."""
+    from generate.batch import BatchEngine
+
+    cfg = make_cfg(MIXED, loop=(0, 2, 2))
+    model, _ = build(cfg, seed=16)
+    V = cfg["vocab"]
+    prompts = [tokens_of(n, V, seed=40 + n) for n in (11, 4, 23)]
+    eng = BatchEngine(model, max_seq_length=48)
+    eager = eng.generate(prompts, 14)
+    for _ in range(2):
+        assert eng.generate(prompts, 14, use_graph=True) == eager
+        assert eng.generate(prompts[::-1], 3) == [e[:len(p) + 3] for e, p in zip(eager[::-1], prompts[::-1])]
+    assert not eng.live
+    # replay by replay against the logits of the eager steps
+    ids = ["x", "y", "z"]
+    logits = eng.step([(i, p, [len(p) - 1]) for i, p in zip(ids, prompts)])
+    first = [int(torch.argmax(logits[i])) for i in range(3)]
+    graph = eng.decode_graph(ids, first)
+    for n in range(6):
+        drawn = graph.step().cpu().tolist()
+        assert drawn == [e[len(p) + 1 + n] for e, p in zip(eager, prompts)], n
+        torch.cuda.synchronize()
+    eng.step([], end=ids)
+
+
 def test_checkpoint_folder_round_trip(tmp_path):
     """config.json + model.safetensors written to a folder: the registry picks the class, the loader the tensors."""
     import json
