@@ -109,6 +109,57 @@ int lgs_token_side(float* x, const int* tokens, const void* table, int w_f32, lo
                    const void* gate_w, const void* proj_w, const float* norm_w, int T, int W, int dim, int vocab,
                    float eps, lgs_stream_t stream);
 
+/* ---- several residual streams (hyper-connections) ---- */
+/* x[t][j] = table[tokens[t]] * scale for each of `streams` streams: x is [T][streams][W] */
+int lgs_embed_streams(const int* tokens, const void* table, int w_f32, float scale, float* x, int T, int W, int vocab,
+                      int streams, lgs_stream_t stream);
+/* One sublayer boundary on x [T][streams][W], in place. With y [T][W] (a sublayer's output):
+ * x_j <- sum_i mix[i * streams + j] x_i + out[j] y. Then, with `in`: u = sum_j in[j] x_j,
+ * h = u / sqrt(mean(u^2) + eps) * norm_w (h_bf16: optional rounded copy), or h = u itself when norm_w is NULL.
+ * Either half may be left out (y or in NULL). streams <= 8; mix / out / in are fp32 on the device. */
+int lgs_streams_step(float* x, const float* y, const float* mix, const float* out, const float* in,
+                     const float* norm_w, float* h, void* h_bf16, float eps, int T, int W, int streams,
+                     lgs_stream_t stream);
+
+/* ---- differential attention ---- */
+/* Per token: rotary (interleaved pairs 2i, 2i + 1 of the first rot_dims dims of every map; angle = position *
+ * inv_freq[i]) on the 2 H query maps at proj[q_off ..] in place and on the 2 G key maps at proj[k_off ..] on their way
+ * to cache_k [slots][max_seq][G][2 d]; the values at proj[v_off ..] go to cache_v [slots][max_seq][G][dv]. The caches
+ * are bf16, or fp32 with cache_f32. k_off < 0: queries only (the layer attends over another layer's cache). */
+int lgs_diffattn_prepare(float* proj, long ld, int q_off, int k_off, int v_off, void* cache_k, void* cache_v,
+                         int cache_f32, const float* inv_freq, const int* slot, const int* pos, int T, int H, int G,
+                         int d, int dv, int rot_dims, int max_seq, lgs_stream_t stream);
+/* out[t][h] = post * unit_rms(a1 - lambda a2), a_m = softmax_j(cap(q_m . k_m,j * scale)) V over the cached rows
+ * lo <= j <= position of the sequence's slot, lo = position - position % chunk (chunk 0: lo = 0);
+ * cap(s) = cap tanh(s / cap) (cap 0: none); query head h reads key head h / (H / G). q: the rotated queries
+ * (row stride ld, 2 d per head). max_len: the most tokens a sequence brings; with max_len 1 the keys of a
+ * (token, head) may be spread over `splits` workgroups (part: T H splits (4 + 2 dv) floats). dv <= 256. */
+int lgs_diffattn(const float* q, long ld, const void* cache_k, const void* cache_v, int cache_f32, const int* seq_start,
+                 const int* seq_slot, const int* seq_pos0, float* out, void* out_bf16, float* part, int splits, int B,
+                 int max_len, int H, int G, int d, int dv, int max_seq, int chunk, float scale, float cap, float lambda,
+                 float eps, float post, lgs_stream_t stream);
+
+/* ---- selective state-space mixer ---- */
+/* out[t][c] = silu(bias[c] + sum_j w[c][j] u[t - (taps - 1 - j)][c]) per sequence of a packed batch; inputs before
+ * the step come from state [slots][taps - 1][C] (oldest first; zeros when the sequence starts at position 0), which
+ * is left holding the step's last taps - 1 inputs. taps <= 16. */
+int lgs_conv_silu(const float* u, long ld, const void* w, const void* bias, int w_f32, float* state,
+                  const int* seq_start, const int* seq_slot, const int* seq_pos0, float* out, int B, int max_len, int C,
+                  int taps, lgs_stream_t stream);
+/* Per sequence and head: dt = softplus(dt_raw + dt_bias), S <- exp(-exp(A_log) dt) S + dt B x^T, y = S^T C + D x.
+ * xbc rows hold x [heads][dv] | B [groups][N] | C [groups][N]; head h reads group h / (heads / groups).
+ * state [slots][heads][N][dv] fp32 is read unless the sequence starts at position 0, and written back. N <= 256. */
+int lgs_ssm_scan(const float* xbc, long ldx, const float* dt, long ldd, const float* dt_bias, const float* A_log,
+                 const float* D, float* state, const int* seq_start, const int* seq_slot, const int* seq_pos0,
+                 float* y, int B, int heads, int groups, int N, int dv, lgs_stream_t stream);
+/* out = v / sqrt(mean over the group of v^2 + eps) * w, v = y * silu(z); `groups` equal parts of `inner` columns */
+int lgs_gated_group_norm(const float* y, const float* z, long ldz, const float* w, float eps, float* out,
+                         void* out_bf16, int T, int inner, int groups, lgs_stream_t stream);
+/* out[t][i] = g sigmoid(alpha g) (u + shift), g = min(a[t ld + i], limit), u = clamp(b[t ld + i], -limit, limit)
+ * (limit <= 0: no clamps) */
+int lgs_glu_clamped(const float* a, const float* b, long ld, void* out, int out_bf16, int T, int n, float alpha,
+                    float limit, float shift, lgs_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

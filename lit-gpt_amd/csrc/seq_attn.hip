@@ -1,0 +1,370 @@
+// Differential attention of the layered models: scores, weights and sums in fp32.
+//
+// A query head carries two maps (q1, q2), a key head two key maps (k1, k2); both maps are softmax attentions over
+// the same values, combined as o = a1 - lambda a2, divided by the head's root mean square and scaled. Query head h
+// reads key/value head h / (H / G). Scores are (q . k) * scale, optionally soft-capped (cap * tanh(s / cap)); a
+// query at position i sees keys lo(i) <= j <= i with lo(i) = i - i % chunk for a chunked mask (chunks are aligned
+// to the sequence's position 0) and 0 without one.
+//
+//   lgs_diffattn_prepare  per token: rotary (interleaved pairs 2i, 2i + 1 of the first rot_dims dims of every map)
+//                         on the queries in place and on the keys on their way into the cache; values into the cache.
+//                         Without key / value columns (a layer that reads another layer's cache) only the queries.
+//   lgs_diffattn          QT consecutive queries of one sequence and one head per workgroup against key tiles of 256
+//                         cached rows: a thread per key for the scores, an online softmax per (query, map), a thread
+//                         per value column for the weighted sums. One query per workgroup (decode) can spread its
+//                         keys over several workgroups, merged by a second launch.
+#include "seq_common.h"
+
+namespace lgs {
+
+struct AttnPrepArgs {
+  float* proj;
+  long ld;
+  int q_off, k_off, v_off;  // k_off < 0: queries only
+  void* cache_k;            // [slots][S][G][2 d]
+  void* cache_v;            // [slots][S][G][dv]
+  const float* inv_freq;    // [rot_dims / 2]
+  const int *slot, *pos;
+  int H, G, d, dv, rot_dims, S;
+};
+
+template <bool CF32>
+__device__ __forceinline__ void cstore(void* c, size_t i, float v) {
+  if (CF32) ((float*)c)[i] = v;
+  else ((uint16_t*)c)[i] = f2bf(v);
+}
+template <bool CF32>
+__device__ __forceinline__ float cload(const void* c, size_t i) {
+  return CF32 ? ((const float*)c)[i] : bf2f(((const uint16_t*)c)[i]);
+}
+
+// grid (T): threads walk (vector, pair) items: 2 H query maps, then 2 G key maps, then the value columns
+template <bool CF32>
+__global__ void __launch_bounds__(256) diffattn_prepare_kernel(AttnPrepArgs p) {
+  const size_t t = blockIdx.x;
+  const int pos = p.pos[t];
+  float* row = p.proj + t * p.ld;
+  const int d = p.d, half = d / 2 + (d & 1), rp = p.rot_dims / 2;
+  const int nq = 2 * p.H * half, nk = p.k_off >= 0 ? 2 * p.G * half : 0;
+  const size_t crow = ((size_t)p.slot[t] * p.S + pos) * p.G;
+  for (int it = threadIdx.x; it < nq + nk; it += 256) {
+    const bool isk = it >= nq;
+    const int e = isk ? it - nq : it;
+    const int vec = e / half, i = e % half;
+    float* src = row + (isk ? p.k_off : p.q_off) + vec * d + 2 * i;
+    const bool pair = 2 * i + 1 < d;
+    float u = src[0], v = pair ? src[1] : 0.0f;
+    if (i < rp) {
+      float sn, cs;
+      sincosf((float)pos * p.inv_freq[i], &sn, &cs);
+      const float nu = u * cs - v * sn, nv = v * cs + u * sn;
+      u = nu;
+      v = nv;
+    }
+    if (isk) {
+      const size_t at = crow * 2 * d + (size_t)vec * d + 2 * i;
+      cstore<CF32>(p.cache_k, at, u);
+      if (pair) cstore<CF32>(p.cache_k, at + 1, v);
+    } else {
+      src[0] = u;
+      if (pair) src[1] = v;
+    }
+  }
+  if (p.k_off >= 0) {
+    const int nv = p.G * p.dv;
+    for (int i = threadIdx.x; i < nv; i += 256) cstore<CF32>(p.cache_v, crow * p.dv + i, row[p.v_off + i]);
+  }
+}
+
+struct AttnArgs {
+  const float* q;  // rotated queries at q + row * ld + h * 2 d
+  long ld;
+  const void* cache_k;
+  const void* cache_v;
+  const int *seq_start, *seq_slot, *seq_pos0;
+  float* out;       // [T][H * dv]
+  uint16_t* out16;  // optional bf16 copy
+  float* part;      // splits > 1: [T][H][splits][4 + 2 dv]
+  int H, G, d, dv, S, chunk, tiles;
+  float scale, cap, lambda, eps, post;
+};
+
+constexpr int kKeyTile = 256;
+
+// o = a1 / l1 - lambda a2 / l2 over the head, unit RMS, times post. Called by all 256 threads; thread c < dv owns
+// column c (dv <= 256).
+__device__ __forceinline__ void diff_finish(float a1, float a2, float l1, float l2, const AttnArgs& p, size_t row, int h,
+                                            float* red) {
+  const int c = threadIdx.x;
+  const float o = c < p.dv ? a1 / l1 - p.lambda * (a2 / l2) : 0.0f;
+  const float ss = block_sum_256(o * o, red);
+  const float v = o / sqrtf(ss / (float)p.dv + p.eps) * p.post;
+  if (c < p.dv) {
+    const size_t at = row * p.H * p.dv + (size_t)h * p.dv + c;
+    p.out[at] = v;
+    if (p.out16) p.out16[at] = f2bf(v);
+  }
+}
+
+// grid (B * tiles, H, splits). LDS: queries [QT][2 d], scores / weights [2 QT][256], per (query, map) the running
+// maximum, normaliser and the rescale of the current tile, and the cross-subset sums of the value phase.
+template <int QT, bool CF32>
+__global__ void __launch_bounds__(256) diffattn_kernel(AttnArgs p) {
+  extern __shared__ float lds[];
+  __shared__ float red[4];
+  const int d = p.d, dv = p.dv, d2 = 2 * d;
+  float* qs = lds;                       // [QT][d2]
+  float* sc = qs + QT * d2;              // [2 QT][kKeyTile]
+  float* mrow = sc + 2 * QT * kKeyTile;  // [2 QT] running maximum
+  float* lrow = mrow + 2 * QT;           // [2 QT] running normaliser
+  float* arow = lrow + 2 * QT;           // [2 QT] rescale of what was summed before this tile
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int b = blockIdx.x / p.tiles, tile = blockIdx.x % p.tiles;
+  const int h = blockIdx.y, g = h / (p.H / p.G);
+  const int r0 = p.seq_start[b] + tile * QT;
+  const int rend = p.seq_start[b + 1];
+  if (r0 >= rend) return;
+  const int nq = min(QT, rend - r0);
+  const int pos_first = p.seq_pos0[b] + tile * QT, pos_last = pos_first + nq - 1;
+  const size_t slot = p.seq_slot[b];
+  const int chunk = p.chunk;
+  int lo = chunk > 0 ? pos_first - pos_first % chunk : 0, hi = pos_last + 1;
+  if (gridDim.z > 1) {  // (QT == 1) an equal share of the keys, in whole numbers
+    const int n = hi - lo, per = (n + gridDim.z - 1) / gridDim.z;
+    lo += blockIdx.z * per;
+    hi = min(hi, lo + per);
+  }
+  for (int i = tid; i < nq * d2; i += 256) qs[i] = p.q[(size_t)(r0 + i / d2) * p.ld + (size_t)h * d2 + i % d2];
+  if (tid < 2 * QT) {
+    mrow[tid] = -INFINITY;
+    lrow[tid] = 0.0f;
+  }
+  // value phase: thread owns column `col` and every KS-th key of a tile, starting at `ks`
+  int ncol = 64;
+  while (ncol < dv) ncol <<= 1;  // dv <= 256
+  const int KS = 256 / ncol, col = tid % ncol, ks = tid / ncol;
+  float acc[QT][2];
+#pragma unroll
+  for (int i = 0; i < QT; ++i) acc[i][0] = acc[i][1] = 0.0f;
+  __syncthreads();
+
+  for (int k0 = lo; k0 < hi; k0 += kKeyTile) {
+    const int nk = min(kKeyTile, hi - k0);
+    // ---- scores of key k0 + tid against every query and map
+    {
+      float s[QT][2];
+#pragma unroll
+      for (int i = 0; i < QT; ++i) s[i][0] = s[i][1] = 0.0f;
+      if (tid < nk) {
+        const size_t kr = ((slot * p.S + k0 + tid) * p.G + g) * d2;
+        if ((d & 3) == 0) {
+          for (int m = 0; m < 2; ++m)
+            for (int e = 0; e < d; e += 4) {
+              float kv[4];
+              if (CF32) {
+                const float4 t4 = *(const float4*)((const float*)p.cache_k + kr + m * d + e);
+                kv[0] = t4.x, kv[1] = t4.y, kv[2] = t4.z, kv[3] = t4.w;
+              } else {
+                const uint2 t2 = *(const uint2*)((const uint16_t*)p.cache_k + kr + m * d + e);
+                kv[0] = bflo(t2.x), kv[1] = bfhi(t2.x), kv[2] = bflo(t2.y), kv[3] = bfhi(t2.y);
+              }
+#pragma unroll
+              for (int i = 0; i < QT; ++i) {
+                const float4 q4 = *(const float4*)(qs + i * d2 + m * d + e);
+                s[i][m] = fmaf(q4.x, kv[0], s[i][m]);
+                s[i][m] = fmaf(q4.y, kv[1], s[i][m]);
+                s[i][m] = fmaf(q4.z, kv[2], s[i][m]);
+                s[i][m] = fmaf(q4.w, kv[3], s[i][m]);
+              }
+            }
+        } else {
+          for (int m = 0; m < 2; ++m)
+            for (int e = 0; e < d; ++e) {
+              const float kv = cload<CF32>(p.cache_k, kr + m * d + e);
+#pragma unroll
+              for (int i = 0; i < QT; ++i) s[i][m] = fmaf(qs[i * d2 + m * d + e], kv, s[i][m]);
+            }
+        }
+      }
+      const int kpos = k0 + tid;
+#pragma unroll
+      for (int i = 0; i < QT; ++i) {
+        const int qpos = pos_first + i;
+        const int qlo = chunk > 0 ? qpos - qpos % chunk : 0;
+        const bool see = tid < nk && i < nq && kpos <= qpos && kpos >= qlo;
+#pragma unroll
+        for (int m = 0; m < 2; ++m) {
+          float v = s[i][m] * p.scale;
+          if (p.cap > 0.0f) v = p.cap * tanhf(v / p.cap);
+          sc[(2 * i + m) * kKeyTile + tid] = see ? v : -INFINITY;
+        }
+      }
+    }
+    __syncthreads();
+    // ---- online softmax: wave w owns rows w, w + 4, ... of the 2 QT (query, map) rows
+    for (int r = wave; r < 2 * QT; r += 4) {
+      float* srow = sc + r * kKeyTile;
+      float v[4], mx = -INFINITY;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        v[e] = srow[lane + 64 * e];
+        mx = fmaxf(mx, v[e]);
+      }
+      mx = wave_max(mx);
+      const float mo = mrow[r], mn = fmaxf(mo, mx);
+      float sum = 0.0f;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float w = mn == -INFINITY ? 0.0f : expf(v[e] - mn);  // (a masked key: exp(-inf) = 0)
+        srow[lane + 64 * e] = w;
+        sum += w;
+      }
+      sum = wave_sum(sum);
+      if (lane == 0) {
+        const float a = mo == -INFINITY ? 0.0f : expf(mo - mn);
+        arow[r] = a;
+        lrow[r] = lrow[r] * a + sum;
+        mrow[r] = mn;
+      }
+    }
+    __syncthreads();
+    // ---- weighted sums of the values
+    {
+#pragma unroll
+      for (int i = 0; i < QT; ++i) {
+        acc[i][0] *= arow[2 * i];
+        acc[i][1] *= arow[2 * i + 1];
+      }
+      if (col < dv) {
+        for (int j = ks; j < nk; j += KS) {
+          const float v = cload<CF32>(p.cache_v, ((slot * p.S + k0 + j) * p.G + g) * dv + col);
+#pragma unroll
+          for (int i = 0; i < QT; ++i) {
+            acc[i][0] = fmaf(sc[(2 * i) * kKeyTile + j], v, acc[i][0]);
+            acc[i][1] = fmaf(sc[(2 * i + 1) * kKeyTile + j], v, acc[i][1]);
+          }
+        }
+      }
+    }
+    __syncthreads();
+  }
+  // ---- sum the key subsets (fixed order), then finish or leave the split's partial result
+  float* xs = sc;  // [KS][2 QT][ncol] <= 256 * 2 QT floats
+  if (KS > 1) {
+#pragma unroll
+    for (int i = 0; i < QT; ++i) {
+      xs[(ks * 2 * QT + 2 * i) * ncol + col] = acc[i][0];
+      xs[(ks * 2 * QT + 2 * i + 1) * ncol + col] = acc[i][1];
+    }
+    __syncthreads();
+  }
+  for (int i = 0; i < nq; ++i) {
+    float a1 = 0.0f, a2 = 0.0f;
+    if (KS > 1) {
+      if (tid < ncol)
+        for (int z = 0; z < KS; ++z) {
+          a1 += xs[(z * 2 * QT + 2 * i) * ncol + tid];
+          a2 += xs[(z * 2 * QT + 2 * i + 1) * ncol + tid];
+        }
+    } else {
+#pragma unroll
+      for (int e = 0; e < QT; ++e)  // (static indexing keeps acc in registers)
+        if (e == i) a1 = acc[e][0], a2 = acc[e][1];
+    }
+    if (gridDim.z > 1) {
+      float* pr = p.part + (((size_t)(r0 + i) * p.H + h) * gridDim.z + blockIdx.z) * (4 + 2 * dv);
+      if (tid == 0) pr[0] = mrow[0], pr[1] = lrow[0], pr[2] = mrow[1], pr[3] = lrow[1];
+      if (tid < dv) pr[4 + tid] = a1, pr[4 + dv + tid] = a2;
+    } else {
+      diff_finish(a1, a2, lrow[2 * i], lrow[2 * i + 1], p, (size_t)(r0 + i), h, red);
+    }
+  }
+}
+
+// grid (T, H): merges the splits of one (token, head) in split order and finishes
+__global__ void __launch_bounds__(256) diffattn_combine_kernel(AttnArgs p, int splits) {
+  __shared__ float red[4];
+  const size_t t = blockIdx.x;
+  const int h = blockIdx.y, dv = p.dv, c = threadIdx.x;
+  const float* pr = p.part + ((t * p.H + h) * splits) * (4 + 2 * dv);
+  float m1 = -INFINITY, m2 = -INFINITY;
+  for (int z = 0; z < splits; ++z) {
+    m1 = fmaxf(m1, pr[(size_t)z * (4 + 2 * dv)]);
+    m2 = fmaxf(m2, pr[(size_t)z * (4 + 2 * dv) + 2]);
+  }
+  float l1 = 0.0f, l2 = 0.0f, a1 = 0.0f, a2 = 0.0f;
+  for (int z = 0; z < splits; ++z) {
+    const float* q = pr + (size_t)z * (4 + 2 * dv);
+    const float w1 = q[0] == -INFINITY ? 0.0f : expf(q[0] - m1), w2 = q[2] == -INFINITY ? 0.0f : expf(q[2] - m2);
+    l1 = fmaf(q[1], w1, l1);
+    l2 = fmaf(q[3], w2, l2);
+    if (c < dv) {
+      a1 = fmaf(q[4 + c], w1, a1);
+      a2 = fmaf(q[4 + dv + c], w2, a2);
+    }
+  }
+  diff_finish(a1, a2, l1, l2, p, t, h, red);
+}
+
+template <int QT>
+static size_t diffattn_lds(int d) { return sizeof(float) * ((size_t)QT * 2 * d + 2 * QT * kKeyTile + 6 * QT); }
+
+template <int QT>
+static int diffattn_launch(const AttnArgs& p, int cache_f32, dim3 grid, hipStream_t stream) {
+  const size_t lds = diffattn_lds<QT>(p.d);
+  auto* fn = cache_f32 ? diffattn_kernel<QT, true> : diffattn_kernel<QT, false>;
+  if (lds > 48 * 1024) {
+    const hipError_t e = hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) {
+      lga_set_error(hipGetErrorString(e));
+      return (int)e;
+    }
+  }
+  fn<<<grid, 256, lds, stream>>>(p);
+  return 0;
+}
+
+}  // namespace lgs
+
+extern "C" int lgs_diffattn_prepare(float* proj, long ld, int q_off, int k_off, int v_off, void* cache_k, void* cache_v,
+                                    int cache_f32, const float* inv_freq, const int* slot, const int* pos, int T, int H,
+                                    int G, int d, int dv, int rot_dims, int max_seq, hipStream_t stream) {
+  LGA_CHECK_ARG(proj && slot && pos && T > 0, "lgs_diffattn_prepare: bad arguments");
+  LGA_CHECK_ARG(H > 0 && G > 0 && H % G == 0 && d > 0 && dv > 0, "lgs_diffattn_prepare: heads must be a multiple of the key heads");
+  LGA_CHECK_ARG(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= d && (rot_dims == 0 || inv_freq),
+                "lgs_diffattn_prepare: rotary dims");
+  LGA_CHECK_ARG(k_off < 0 || (cache_k && cache_v && v_off >= 0 && max_seq > 0), "lgs_diffattn_prepare: cache");
+  LGA_CHECK_ARG(q_off >= 0 && q_off + 2L * H * d <= ld, "lgs_diffattn_prepare: queries outside the row");
+  LGA_CHECK_ARG(k_off < 0 || (k_off + 2L * G * d <= ld && v_off + (long)G * dv <= ld),
+                "lgs_diffattn_prepare: keys or values outside the row");
+  lgs::AttnPrepArgs p{proj, ld, q_off, k_off, v_off, cache_k, cache_v, inv_freq, slot, pos, H, G, d, dv, rot_dims, max_seq};
+  if (cache_f32) lgs::diffattn_prepare_kernel<true><<<T, 256, 0, stream>>>(p);
+  else lgs::diffattn_prepare_kernel<false><<<T, 256, 0, stream>>>(p);
+  LGA_LAUNCH_RETURN();
+}
+
+extern "C" int lgs_diffattn(const float* q, long ld, const void* cache_k, const void* cache_v, int cache_f32,
+                            const int* seq_start, const int* seq_slot, const int* seq_pos0, float* out, void* out_bf16,
+                            float* part, int splits, int B, int max_len, int H, int G, int d, int dv, int max_seq,
+                            int chunk, float scale, float cap, float lambda, float eps, float post, hipStream_t stream) {
+  LGA_CHECK_ARG(q && cache_k && cache_v && seq_start && seq_slot && seq_pos0 && out, "lgs_diffattn: null pointer");
+  LGA_CHECK_ARG(B > 0 && max_len > 0 && H > 0 && H <= 65535 && G > 0 && H % G == 0, "lgs_diffattn: bad sizes");
+  LGA_CHECK_ARG(d > 0 && d <= 512 && dv > 0 && dv <= 256, "lgs_diffattn: key dim <= 512, value dim <= 256");
+  LGA_CHECK_ARG(ld >= 2L * H * d && chunk >= 0 && max_seq > 0, "lgs_diffattn: bad sizes");
+  LGA_CHECK_ARG(splits >= 1 && splits <= 64 && (splits == 1 || (part && max_len == 1)),
+                "lgs_diffattn: splits need one token per sequence and a workspace");
+  lgs::AttnArgs p{q, ld, cache_k, cache_v, seq_start, seq_slot, seq_pos0, out, (uint16_t*)out_bf16, part,
+                  H, G, d, dv, max_seq, chunk, 0, scale, cap, lambda, eps, post};
+  int rc;
+  if (max_len == 1) {
+    p.tiles = 1;
+    rc = lgs::diffattn_launch<1>(p, cache_f32, dim3(B, H, splits), stream);
+    if (rc == 0 && splits > 1) lgs::diffattn_combine_kernel<<<dim3(B, H), 256, 0, stream>>>(p, splits);
+  } else {
+    p.tiles = (max_len + 7) / 8;
+    LGA_CHECK_ARG((long)B * p.tiles < (1L << 31), "lgs_diffattn: too many tiles");
+    rc = lgs::diffattn_launch<8>(p, cache_f32, dim3(B * p.tiles, H, 1), stream);
+  }
+  if (rc) return rc;
+  LGA_LAUNCH_RETURN();
+}

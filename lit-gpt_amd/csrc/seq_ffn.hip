@@ -1,6 +1,7 @@
 // Feed-forward parts of the layered models.
 //
 //   lgs_glu              out = act(a) * b over two column ranges of one projection (the dense gated feed-forward)
+//   lgs_glu_clamped      out = g sigmoid(alpha g) (u + shift) with g = min(a, limit), u = clamp(b, -limit, limit)
 //   lgs_moe_route        per token: the `top` largest router logits (fp32, lowest index first among equals) and the
 //                        softmax over just those
 //   lgs_moe_up / _down   the routed experts as streaming GEMVs over (token, choice) pairs: only the chosen experts'
@@ -20,6 +21,24 @@ __global__ void __launch_bounds__(256) glu_kernel(const float* __restrict__ a, c
   if (i >= n) return;
   const float v = act_f(act, a[t * ld + i]) * b[t * ld + i];
   if (out16) out16[t * n + i] = f2bf(v);  // the operand of a bf16 product: rounded here instead of at its load
+  else out[t * n + i] = v;
+}
+
+// grid (T, ceil(n / 256)): g = min(a, limit), u = clamp(b, -limit, limit); out = g sigmoid(alpha g) (u + shift)
+// (limit <= 0: no clamps)
+__global__ void __launch_bounds__(256) glu_clamped_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                          long ld, float* __restrict__ out, uint16_t* __restrict__ out16,
+                                                          int n, float alpha, float limit, float shift) {
+  const size_t t = blockIdx.x;
+  const int i = blockIdx.y * 256 + threadIdx.x;
+  if (i >= n) return;
+  float g = a[t * ld + i], u = b[t * ld + i];
+  if (limit > 0.0f) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+  }
+  const float v = g * sigmoid_f(alpha * g) * (u + shift);
+  if (out16) out16[t * n + i] = f2bf(v);
   else out[t * n + i] = v;
 }
 
@@ -231,6 +250,14 @@ extern "C" int lgs_glu(const float* a, const float* b, long ld, void* out, int o
   LGA_CHECK_ARG(a && b && out && T > 0 && T <= 65535 && n > 0, "lgs_glu: bad arguments");
   lgs::glu_kernel<<<dim3((n + 255) / 256, T), 256, 0, stream>>>(a, b, ld, out_bf16 ? nullptr : (float*)out,
                                                                  out_bf16 ? (uint16_t*)out : nullptr, n, act);
+  LGA_LAUNCH_RETURN();
+}
+
+extern "C" int lgs_glu_clamped(const float* a, const float* b, long ld, void* out, int out_bf16, int T, int n,
+                               float alpha, float limit, float shift, hipStream_t stream) {
+  LGA_CHECK_ARG(a && b && out && T > 0 && n > 0 && (n + 255) / 256 <= 65535, "lgs_glu_clamped: bad arguments");
+  lgs::glu_clamped_kernel<<<dim3(T, (n + 255) / 256), 256, 0, stream>>>(
+      a, b, ld, out_bf16 ? nullptr : (float*)out, out_bf16 ? (uint16_t*)out : nullptr, n, alpha, limit, shift);
   LGA_LAUNCH_RETURN();
 }
 

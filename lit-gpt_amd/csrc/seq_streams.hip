@@ -1,0 +1,118 @@
+// Multi-stream residual (hyper-connections) of the layered models, fp32 throughout.
+//
+// The residual is kept in `s` parallel streams x[t][0 .. s)[W]. A sublayer reads a fixed weighted sum of the
+// streams, u = sum_i a[i] x_i, through an RMS norm; its output y goes back into every stream while the streams
+// are mixed: x_j <- sum_i m[i][j] x_i + b[j] y. With s = 1, a = b = m = 1 this is the ordinary residual sum.
+//
+//   lgs_embed_streams   x[t][j] = table[tokens[t]] * scale for every stream j
+//   lgs_streams_step    one launch per sublayer boundary: the write-back of the sublayer that just ran (optional)
+//                       followed by the read + norm of the next one (optional), so the streams are read once
+#include "seq_common.h"
+
+namespace lgs {
+
+constexpr int kMaxStreams = 8;
+
+template <bool WF32>
+__global__ void __launch_bounds__(256) embed_streams_kernel(const int* __restrict__ tokens, const void* __restrict__ table,
+                                                            float scale, float* __restrict__ x, int W, int streams) {
+  const size_t t = blockIdx.x;
+  const size_t src = (size_t)tokens[t] * W;
+  for (int i = threadIdx.x; i < W; i += 256) {
+    const float v = wload<WF32>(table, src + i) * scale;
+    for (int j = 0; j < streams; ++j) x[(t * streams + j) * W + i] = v;
+  }
+}
+
+struct StreamArgs {
+  float* x;          // [T][s][W]
+  const float* y;    // [T][W] sublayer output to write back (null: no write-back)
+  const float* mix;  // [s][s] indexed [from][to]
+  const float* out;  // [s]
+  const float* in;   // [s] read weights of the next sublayer (null: no read)
+  const float* w;    // [W] norm weight of the next sublayer (null: the weighted sum itself is the result)
+  float* h;          // [T][W] normed read
+  uint16_t* h16;     // optional bf16 copy of h
+  float eps;
+  int W, s;
+};
+
+// grid (T): a workgroup owns a token; thread i owns columns i, i + 256, ... in every stream
+__global__ void __launch_bounds__(256) streams_step_kernel(StreamArgs p) {
+  __shared__ float red[4];
+  __shared__ float cm[kMaxStreams * kMaxStreams], cb[kMaxStreams], ca[kMaxStreams];
+  const int s = p.s, W = p.W;
+  if (threadIdx.x < s * s) cm[threadIdx.x] = p.mix ? p.mix[threadIdx.x] : 0.0f;
+  if (threadIdx.x < s) {
+    cb[threadIdx.x] = p.out ? p.out[threadIdx.x] : 0.0f;
+    ca[threadIdx.x] = p.in ? p.in[threadIdx.x] : 0.0f;
+  }
+  __syncthreads();
+  float* xt = p.x + (size_t)blockIdx.x * s * W;
+  const float* yt = p.y ? p.y + (size_t)blockIdx.x * W : nullptr;
+  float ss = 0.0f;
+  for (int i = threadIdx.x; i < W; i += 256) {
+    float v[kMaxStreams];
+#pragma unroll
+    for (int j = 0; j < kMaxStreams; ++j) v[j] = j < s ? xt[(size_t)j * W + i] : 0.0f;
+    if (yt) {
+      const float y = yt[i];
+      float nv[kMaxStreams];
+#pragma unroll
+      for (int j = 0; j < kMaxStreams; ++j) {
+        float acc = 0.0f;
+#pragma unroll
+        for (int k = 0; k < kMaxStreams; ++k)
+          if (k < s && j < s) acc = fmaf(cm[k * s + j], v[k], acc);
+        nv[j] = j < s ? fmaf(cb[j], y, acc) : 0.0f;
+      }
+#pragma unroll
+      for (int j = 0; j < kMaxStreams; ++j) {
+        v[j] = nv[j];
+        if (j < s) xt[(size_t)j * W + i] = nv[j];
+      }
+    }
+    if (p.in) {
+      float u = 0.0f;
+#pragma unroll
+      for (int j = 0; j < kMaxStreams; ++j)
+        if (j < s) u = fmaf(ca[j], v[j], u);
+      ss = fmaf(u, u, ss);
+      p.h[(size_t)blockIdx.x * W + i] = u;  // normed below
+    }
+  }
+  if (!p.in || !p.w) return;
+  ss = block_sum_256(ss, red);
+  const float rstd = 1.0f / sqrtf(ss / (float)W + p.eps);
+  for (int i = threadIdx.x; i < W; i += 256) {
+    const size_t at = (size_t)blockIdx.x * W + i;
+    const float v = p.h[at] * rstd * p.w[i];  // (each thread re-reads what it wrote itself)
+    p.h[at] = v;
+    if (p.h16) p.h16[at] = f2bf(v);
+  }
+}
+
+}  // namespace lgs
+
+extern "C" int lgs_embed_streams(const int* tokens, const void* table, int w_f32, float scale, float* x, int T, int W,
+                                 int vocab, int streams, hipStream_t stream) {
+  LGA_CHECK_ARG(tokens && table && x && T > 0 && W > 0 && vocab > 0, "lgs_embed_streams: bad arguments");
+  LGA_CHECK_ARG(streams >= 1 && streams <= lgs::kMaxStreams, "lgs_embed_streams: 1 to 8 streams");
+  if (w_f32) lgs::embed_streams_kernel<true><<<T, 256, 0, stream>>>(tokens, table, scale, x, W, streams);
+  else lgs::embed_streams_kernel<false><<<T, 256, 0, stream>>>(tokens, table, scale, x, W, streams);
+  LGA_LAUNCH_RETURN();
+}
+
+extern "C" int lgs_streams_step(float* x, const float* y, const float* mix, const float* out, const float* in,
+                                const float* norm_w, float* h, void* h_bf16, float eps, int T, int W, int streams,
+                                hipStream_t stream) {
+  LGA_CHECK_ARG(x && T > 0 && W > 0, "lgs_streams_step: bad arguments");
+  LGA_CHECK_ARG(streams >= 1 && streams <= lgs::kMaxStreams, "lgs_streams_step: 1 to 8 streams");
+  LGA_CHECK_ARG(!y || (mix && out), "lgs_streams_step: a write-back needs the mix matrix and the output weights");
+  LGA_CHECK_ARG(!in || h, "lgs_streams_step: a read needs a result buffer");
+  LGA_CHECK_ARG(norm_w || !h_bf16, "lgs_streams_step: the bf16 copy is made by the norm");
+  LGA_CHECK_ARG(y || in, "lgs_streams_step: nothing to do");
+  lgs::StreamArgs p{x, y, mix, out, in, norm_w, h, (uint16_t*)h_bf16, eps, W, streams};
+  lgs::streams_step_kernel<<<T, 256, 0, stream>>>(p);
+  LGA_LAUNCH_RETURN();
+}

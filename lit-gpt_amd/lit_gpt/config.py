@@ -178,15 +178,24 @@ class RotarySpec:
 
 @dataclass
 class MixerSpec:
-    kind: str  # "retention" | "latent_attention"
+    kind: str  # "retention" | "latent_attention" | "attention" | "mamba2"
     heads: int
-    dim: int  # per-head query / key size (latent attention: the unrotated part)
+    dim: int  # per-head query / key size (latent attention: the unrotated part; attention: of one map)
     vdim: int
     rot: RotarySpec
     decay: Optional[List[float]] = None  # retention: one fixed decay per head
     kv_rank: int = 0  # latent attention: size of the cached latent
     rot_dim: int = 0  # latent attention: rotated query / key part (one key part shared by the heads)
-    scale: float = 1.0  # latent attention: score scale
+    scale: float = 1.0  # attention score scale
+    kv_heads: int = 0  # attention: key / value heads (query head h reads head h // (heads // kv_heads))
+    diff: float = 0.0  # differential attention: the constant of lambda; the output is scaled by 1 - diff
+    softcap: float = 0.0  # attention: scores pass cap * tanh(s / cap) (0: not)
+    mask_size: int = 0  # attention: a query sees keys of its own aligned chunk of this many positions (0: all before it)
+    kv_from: Optional[int] = None  # attention: the layer whose cached keys and values this layer reads
+    conv: int = 0  # mamba2: taps of the short convolution
+    groups: int = 0  # mamba2: groups of heads that share B and C
+    norm_groups: int = 1  # mamba2: equal parts of the gated output, each divided by its own root mean square
+    state: int = 0  # mamba2: state size N
 
 
 @dataclass
@@ -195,6 +204,7 @@ class FeedForwardSpec:
     ff: int
     experts: int = 0
     top: int = 0
+    limit: float = 0.0  # clamped gated unit: bound of the gate (from above) and of the up branch (both sides)
 
 
 @dataclass
@@ -203,7 +213,23 @@ class LayerSpec:
     mlp: Optional[FeedForwardSpec]
 
 
-MIXER_KINDS = ("retention", "latent_attention")
+MIXER_KINDS = ("retention", "latent_attention", "attention", "mamba2")
+
+
+@dataclass(frozen=True)
+class LayeredDesign:
+    """What a design fixes for all its models (everything else is in ``config.json``)."""
+
+    block: str  # "parallel": x += mixer(h) + ff(h), one norm; "sequential": x += mixer(norm1 x), then x += ff(norm2 x)
+    norm_offset: float  # the norm multiplies by offset + stored weight
+    tied_head: bool  # logits from the embedding table itself, or from a matrix of their own ("head")
+    dense_ff: str  # "gelu_tanh": W_down(gelu_tanh(gate) * up); "clamped_swish": g sigmoid(1.702 g) (u + 1), clamped
+
+
+DESIGNS: Dict[str, LayeredDesign] = {
+    "Bavesun": LayeredDesign("parallel", 1.0, True, "gelu_tanh"),
+    "Rigulorn": LayeredDesign("sequential", 0.0, False, "clamped_swish"),
+}
 
 
 @dataclass
@@ -219,9 +245,19 @@ class LayeredConfig:
     loop_times: int = 1
     side_dim: int = 0  # per-layer token input: width of each layer's slice of the second embedding table (0: none)
     name: str = ""
+    streams: int = 1  # parallel residual streams (hyper-connections); 1 with no stream weights: the plain residual sum
+    stream_weights: bool = False  # the checkpoint holds read / write / mix weights per sublayer
+
+    @property
+    def design(self) -> LayeredDesign:
+        return DESIGNS[self.architecture]
 
     def __post_init__(self) -> None:
         self.name = self.name or self.architecture
+        if self.architecture not in DESIGNS:
+            raise ValueError(f"architecture {self.architecture!r} is not registered (known: {sorted(DESIGNS)})")
+        if not 1 <= self.streams <= 8:
+            raise ValueError(f"{self.streams} residual streams: 1 to 8 are served")
         n = len(self.layers)
         if not (0 <= self.loop_start <= self.loop_stop <= n) or self.loop_times < 1:
             raise ValueError(f"loop [{self.loop_start}, {self.loop_stop}) x {self.loop_times} does not fit {n} layers")
@@ -231,8 +267,24 @@ class LayeredConfig:
                 raise ValueError(f"layer {i}: unknown mixer {m.kind!r}")
             if m.kind == "retention" and (m.decay is None or len(m.decay) != m.heads):
                 raise ValueError(f"layer {i}: retention needs one decay per head")
+            if m.kind == "mamba2":
+                if m.groups < 1 or m.heads % m.groups or m.norm_groups < 1 or (m.heads * m.vdim) % m.norm_groups:
+                    raise ValueError(f"layer {i}: heads {m.heads} / groups {m.groups} / norm groups {m.norm_groups}")
+                if not (1 <= m.conv <= 16 and 1 <= m.state <= 256):
+                    raise ValueError(f"layer {i}: convolution taps 1..16 and state size 1..256 are served")
+                continue
             if m.rot.dims % 2 or m.rot.dims > (m.rot_dim if m.kind == "latent_attention" else m.dim):
                 raise ValueError(f"layer {i}: rotary dims {m.rot.dims} do not fit the head")
+            if m.kind == "attention":
+                if m.kv_heads < 1 or m.heads % m.kv_heads or m.mask_size < 0 or m.vdim > 256:
+                    raise ValueError(f"layer {i}: heads {m.heads} / key heads {m.kv_heads} / value dim {m.vdim}")
+                if m.kv_from is not None:
+                    j = m.kv_from
+                    src = self.layers[j].mixer if 0 <= j < i else None
+                    if src is None or src.kind != "attention" or src.kv_from is not None:
+                        raise ValueError(f"layer {i}: kv_from {j} must name an earlier attention layer with keys of its own")
+                    if (src.kv_heads, src.dim, src.vdim) != (m.kv_heads, m.dim, m.vdim):
+                        raise ValueError(f"layer {i}: its key heads and sizes differ from layer {j}'s")
             if spec.mlp is not None and spec.mlp.kind == "moe" and not 0 < spec.mlp.top <= spec.mlp.experts:
                 raise ValueError(f"layer {i}: top {spec.mlp.top} of {spec.mlp.experts} experts")
 
@@ -249,16 +301,22 @@ class LayeredConfig:
         for entry in d["layers"]:
             m = entry["mixer"]
             rot = m.get("rot") or {}
-            mixer = MixerSpec(kind=entry["type"], heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+            mask = m.get("mask") or {}
+            mixer = MixerSpec(kind=entry["type"], heads=int(m["heads"]), dim=int(m.get("dim", 0)), vdim=int(m["vdim"]),
                               rot=RotarySpec(int(rot.get("dims", 0)), float(rot.get("base", 10000.0))),
                               decay=[float(x) for x in m["decay"]] if "decay" in m else None,
                               kv_rank=int(m.get("kv_rank", 0)), rot_dim=int(m.get("rot_dim", 0)),
-                              scale=float(m.get("scale", 1.0)))
+                              scale=float(m.get("scale", 1.0)), kv_heads=int(m.get("kv_heads", m["heads"])),
+                              diff=float(m.get("diff", 0.0)), softcap=float(m.get("softcap") or 0.0),
+                              mask_size=int(mask.get("size") or 0),
+                              kv_from=int(m["kv_from"]) if m.get("kv_from") is not None else None,
+                              conv=int(m.get("conv", 0)), groups=int(m.get("groups", 0)),
+                              norm_groups=int(m.get("norm_groups", 1)), state=int(m.get("state", 0)))
             f = entry.get("mlp")
             if f is None:
                 mlp = None
             elif f["kind"] == "dense":
-                mlp = FeedForwardSpec("dense", int(f["ff"]))
+                mlp = FeedForwardSpec("dense", int(f["ff"]), limit=float(f.get("limit") or 0.0))
             elif f["kind"] == "moe":
                 mlp = FeedForwardSpec("moe", int(f["expert"]["ff"]), int(f["router"]["experts"]), int(f["router"]["top"]))
             else:
@@ -269,7 +327,8 @@ class LayeredConfig:
         return cls(architecture=d["architecture"], vocab=int(d["vocab"]), width=int(d["width"]),
                    norm_eps=float(d["norm"]["eps"]), embedding_scale=float((d.get("embedding") or {}).get("scale", 1.0)),
                    layers=layers, loop_start=int(loop.get("start", 0)), loop_stop=int(loop.get("stop", 0)),
-                   loop_times=int(loop.get("times", 1)), side_dim=int(side.get("dim", 0)))
+                   loop_times=int(loop.get("times", 1)), side_dim=int(side.get("dim", 0)),
+                   streams=int(d.get("streams", 1)), stream_weights="streams" in d)
 
     @classmethod
     def from_json(cls, path: Union[str, Path]) -> "LayeredConfig":
@@ -278,7 +337,7 @@ class LayeredConfig:
 
 
 # architecture name (config.json) -> "module:class" of the model that serves it
-ARCHITECTURES: Dict[str, str] = {"Bavesun": "lit_gpt.layered:LayeredGPT"}
+ARCHITECTURES: Dict[str, str] = {"Bavesun": "lit_gpt.layered:LayeredGPT", "Rigulorn": "lit_gpt.layered:LayeredGPT"}
 
 
 def load_config(checkpoint_dir: Union[str, Path]) -> Union[Config, LayeredConfig]:

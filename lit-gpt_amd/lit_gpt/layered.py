@@ -7,9 +7,16 @@ step (``forward_step`` / ``logits``) that ``generate.batch.BatchEngine`` schedul
 attention scores, recurrent states and routers are fp32 in both precisions; ``dtype`` (bf16 or fp32) is the dtype
 of the weight matrices and of the cached latent, and picks bf16-operand / fp32-sum products or plain fp32 ones.
 
-A layer is parallel: h = norm(x); x <- x + mixer(h) + ff(h); then the optional per-layer token input. The norm's
-weight is stored around zero (offset 1). Every matrix that reads h is one row block of a single fused input
-projection. Logits come from the embedding table itself (tied, unscaled) after the final norm.
+The design named by ``config.architecture`` fixes the layer's shape (``config.design``):
+
+* parallel — h = norm(x); x <- x + mixer(h) + ff(h); then the optional per-layer token input. The norm's weight is
+  stored around zero (offset 1); every matrix that reads h is one row block of a single fused input projection;
+  logits come from the embedding table itself (tied, unscaled) after the final norm.
+* sequential — pre-norm sublayers, x <- x + mixer(norm1 x), then x <- x + ff(norm2 x) (a layer may have no
+  feed-forward), over ``config.streams`` parallel residual streams: a sublayer reads a weighted sum of the streams
+  and its output is written into all of them while a small matrix mixes them (``lit_gpt.mixers.StreamLinks``; one
+  stream with unit weights is the plain residual sum). The write-back of a sublayer and the read + norm of the next
+  run as one launch. Logits from a matrix of their own (``head``) after the final norm of the streams' sum.
 """
 
 from __future__ import annotations
@@ -22,7 +29,7 @@ import torch.nn as nn
 
 from lit_gpt import seq_ops
 from lit_gpt.config import LayeredConfig, LayerSpec
-from lit_gpt.mixers import MIXERS, GatedFeedForward, SparseFeedForward, StepBatch, TokenSide
+from lit_gpt.mixers import MIXERS, GatedFeedForward, SparseFeedForward, StepBatch, StreamLinks, TokenSide
 from lit_gpt.rmsnorm import StreamRMSNorm
 
 
@@ -79,6 +86,77 @@ class LayeredBlock(nn.Module):
             self.side(x, step.tokens)
 
 
+def _fuse_rows(parts, width: int, device, dtype) -> Tuple[torch.Tensor, Dict[str, int]]:
+    """Row-wise concatenation of the matrices that read one norm output, every part on a 32-byte boundary of the
+    fp32 result row; returns the matrix and each part's first row."""
+    rows, offsets, at = [], {}, 0
+    for name, t in parts:
+        offsets[name] = at
+        rows.append(t)
+        at += t.shape[0]
+        pad = -at % 8
+        if pad:
+            rows.append(torch.zeros(pad, width, dtype=t.dtype))
+            at += pad
+    return torch.cat(rows).to(device=device, dtype=dtype).contiguous(), offsets
+
+
+class Sublayer(nn.Module):
+    """One pre-norm sublayer of a sequential layer: its norm weight, its links to the residual streams, its fused
+    input projection and the module (a mixer or a feed-forward) that turns the projection into the output."""
+
+    def __init__(self, module: nn.Module, norm_w: torch.Tensor, links: StreamLinks, width: int, device, dtype) -> None:
+        super().__init__()
+        self.module, self.links = module, links
+        self.register_buffer("norm_w", norm_w.to(device=device, dtype=torch.float32).contiguous())
+        w_in, offsets = _fuse_rows(module.in_parts(), width, device, dtype)
+        module.bind(offsets)
+        self.register_buffer("w_in", w_in)
+
+    def wants_bf16(self, rows: int) -> bool:
+        """Whether the norm that feeds this sublayer should also leave a bf16 copy (bf16 MFMA tiles read it)."""
+        return rows > 8 and self.w_in.dtype == torch.bfloat16
+
+    def forward(self, h: torch.Tensor, h16: Optional[torch.Tensor], step: StepBatch, cache) -> torch.Tensor:
+        """h (T, width): the normed read of the streams. Returns the sublayer's output (T, width) fp32."""
+        n_in, W = self.w_in.shape
+        proj = torch.empty(step.T, n_in, dtype=torch.float32, device=h.device)
+        seq_ops.linear(h if h16 is None else h16, self.w_in, M=step.T, N=n_in, K=W, y=proj, lda=W, ldy=n_in)
+        y = torch.empty(step.T, W, dtype=torch.float32, device=h.device)
+        if cache is None:
+            self.module(proj, h, y, h16=h16, accumulate=False)
+        else:
+            self.module(proj, step, cache, y, accumulate=False)
+        return y
+
+
+class SequentialBlock(nn.Module):
+    """A pre-norm layer: the mixer sublayer, then the feed-forward sublayer if the layer has one."""
+
+    def __init__(self, index: int, spec: LayerSpec, config: LayeredConfig, w: Dict[str, torch.Tensor], device,
+                 dtype) -> None:
+        super().__init__()
+        W, eps, design = config.width, config.norm_eps, config.design
+        if design.norm_offset != 0.0:
+            raise NotImplementedError("sequential layers take the norm weight as stored")
+
+        def links(q: int) -> StreamLinks:
+            return StreamLinks(config.streams, _sub(w, f"hc{q}.") if config.stream_weights else None, device)
+
+        self.mixer = MIXERS[spec.mixer.kind](spec.mixer, W, eps, _sub(w, "mix."), device, dtype)
+        self.sub1 = Sublayer(self.mixer, w["norm1"], links(1), W, device, dtype)
+        self.sub2 = None
+        if spec.mlp is not None:
+            if spec.mlp.kind != "dense":
+                raise NotImplementedError("sequential layers serve dense feed-forwards")
+            clamp = (1.702, spec.mlp.limit, 1.0) if design.dense_ff == "clamped_swish" else None
+            mlp = GatedFeedForward(spec.mlp, W, _sub(w, "mlp."), device, dtype, clamp=clamp)
+            self.sub2 = Sublayer(mlp, w["norm2"], links(2), W, device, dtype)
+
+    def sublayers(self) -> List[Sublayer]:
+        return [self.sub1] if self.sub2 is None else [self.sub1, self.sub2]
+
+
 class LayeredGPT(nn.Module):
     decode_graph = False  # generate.base.generate steps this model eagerly (its graph executor is GPT's)
 
@@ -100,10 +178,26 @@ class LayeredGPT(nn.Module):
             if t.shape[0] != V or t.shape[1] < config.side_dim * len(config.layers):
                 raise ValueError(f"side.embed: shape {tuple(t.shape)} does not hold {len(config.layers)} slices")
             self.side_embed = t.to(device=device, dtype=dtype).contiguous()
-        self.blocks = nn.ModuleList(
-            LayeredBlock(i, spec, config, _sub(weights, f"l{i}."), self.side_embed, device, dtype)
-            for i, spec in enumerate(config.layers))
-        self.final_norm = StreamRMSNorm(W, eps=config.norm_eps, offset=1.0)
+        design = config.design
+        self.sequential = design.block == "sequential"
+        if self.sequential:
+            if config.side_dim:
+                raise NotImplementedError("per-layer token inputs belong to the parallel layers")
+            self.blocks = nn.ModuleList(SequentialBlock(i, spec, config, _sub(weights, f"l{i}."), device, dtype)
+                                        for i, spec in enumerate(config.layers))
+            self.register_buffer("stream_ones", torch.ones(config.streams, dtype=torch.float32, device=device))
+        else:
+            if config.streams != 1:
+                raise NotImplementedError("several residual streams belong to the sequential layers")
+            self.blocks = nn.ModuleList(
+                LayeredBlock(i, spec, config, _sub(weights, f"l{i}."), self.side_embed, device, dtype)
+                for i, spec in enumerate(config.layers))
+        self.register_buffer("head", None)
+        if not design.tied_head:
+            if tuple(weights["head"].shape) != (V, W):
+                raise ValueError(f"head: shape {tuple(weights['head'].shape)}, expected {(V, W)}")
+            self.head = weights["head"].to(device=device, dtype=dtype).contiguous()
+        self.final_norm = StreamRMSNorm(W, eps=config.norm_eps, offset=design.norm_offset)
         self.final_norm.weight = weights["final.norm"].to(device=device, dtype=torch.float32).contiguous()
         self.runs: List[int] = config.layer_runs
         self.caches: Optional[nn.ModuleList] = None  # one cache / state per layer run
@@ -124,15 +218,33 @@ class LayeredGPT(nn.Module):
     def tensor_shapes(config: LayeredConfig) -> Dict[str, Tuple[int, ...]]:
         """Name -> shape of every checkpoint tensor of a configuration."""
         W, out = config.width, {"embed": (config.vocab, config.width), "final.norm": (config.width,)}
+        if not config.design.tied_head:
+            out["head"] = (config.vocab, config.width)
         if config.side_dim:
             out["side.embed"] = (config.vocab, config.side_dim * len(config.layers))
         for i, spec in enumerate(config.layers):
             m, p = spec.mixer, f"l{i}."
             out[p + "norm1"] = (W,)
+            if spec.mlp is not None and config.design.block == "sequential":
+                out[p + "norm2"] = (W,)
+            if config.stream_weights:
+                for q in (1, 2) if spec.mlp is not None else (1,):
+                    s = config.streams
+                    out.update({p + f"hc{q}.in": (s,), p + f"hc{q}.out": (s,), p + f"hc{q}.mix": (s, s)})
             if m.kind == "retention":
                 out.update({p + "mix.q": (m.heads * m.dim, W), p + "mix.k": (m.heads * m.dim, W),
                             p + "mix.v": (m.heads * m.vdim, W), p + "mix.g": (m.heads * m.vdim, W),
                             p + "mix.o": (W, m.heads * m.vdim)})
+            elif m.kind == "attention":
+                out.update({p + "mix.q": (2 * m.heads * m.dim, W), p + "mix.o": (W, m.heads * m.vdim)})
+                if m.kv_from is None:
+                    out.update({p + "mix.k": (2 * m.kv_heads * m.dim, W), p + "mix.v": (m.kv_heads * m.vdim, W)})
+                out.update({p + f"mix.{n}": (m.dim,) for n in ("lq1", "lk1", "lq2", "lk2")})
+            elif m.kind == "mamba2":
+                inner, bc = m.heads * m.vdim, 2 * m.groups * m.state
+                out.update({p + "mix.in": (2 * inner + bc + m.heads, W), p + "mix.conv": (inner + bc, m.conv),
+                            p + "mix.conv.b": (inner + bc,), p + "mix.dt_bias": (m.heads,), p + "mix.A_log": (m.heads,),
+                            p + "mix.D": (m.heads,), p + "mix.norm": (inner,), p + "mix.o": (W, inner)})
             else:
                 out.update({p + "mix.q": (m.heads * (m.dim + m.rot_dim), W), p + "mix.dkv": (m.kv_rank + m.rot_dim, W),
                             p + "mix.dkv.norm": (m.kv_rank,), p + "mix.uk": (m.heads * m.dim, m.kv_rank),
@@ -152,12 +264,29 @@ class LayeredGPT(nn.Module):
 
     @classmethod
     def random_weights(cls, config: LayeredConfig, seed: int = 0) -> Dict[str, torch.Tensor]:
-        """Random bf16 checkpoint tensors (matrices ~ N(0, 1/fan_in), norm weights small, sinks ~ N(0, 1))."""
+        """Random bf16 checkpoint tensors (matrices ~ N(0, 1/fan_in), norm weights around the design's neutral value,
+        sinks ~ N(0, 1), stream weights around the plain residual sum, step sizes and decays in a usable range)."""
         g = torch.Generator().manual_seed(seed)
         out = {}
+        neutral = 1.0 - config.design.norm_offset
         for name, shape in cls.tensor_shapes(config).items():
-            if name.endswith("norm1") or name == "final.norm":
-                t = 0.1 * torch.randn(shape, generator=g)
+            leaf = name.rsplit(".", 1)[-1]
+            if leaf in ("norm1", "norm2") or name == "final.norm":
+                t = neutral + 0.1 * torch.randn(shape, generator=g)
+            elif ".hc" in name:
+                s = config.streams
+                t = {"in": torch.full(shape, 1.0 / s), "out": torch.ones(shape), "mix": torch.eye(s)}[leaf] + \
+                    0.2 * torch.randn(shape, generator=g)
+            elif leaf in ("lq1", "lk1", "lq2", "lk2"):
+                t = 0.3 * torch.randn(shape, generator=g)
+            elif leaf == "A_log":
+                t = torch.log(1.0 + 3.0 * torch.rand(shape, generator=g))
+            elif leaf == "dt_bias":
+                t = -2.0 + torch.randn(shape, generator=g)
+            elif leaf == "D":
+                t = 1.0 + 0.2 * torch.randn(shape, generator=g)
+            elif name.endswith("conv.b"):
+                t = 0.2 * torch.randn(shape, generator=g)
             elif name.endswith(".norm"):
                 t = 1.0 + 0.1 * torch.randn(shape, generator=g)
             elif name.endswith("sink"):
@@ -187,9 +316,17 @@ class LayeredGPT(nn.Module):
             self.max_seq_length = max_seq_length
         if self._max_seq_length <= 0:
             raise ValueError("set max_seq_length (or pass it) before set_kv_cache")
-        self.caches = nn.ModuleList(
-            self.blocks[i].mixer.build_cache(batch_size, self._max_seq_length, device or self.device,
-                                             dtype or self.dtype) for i in self.runs)
+        caches, of_layer = [], {}
+        for i in self.runs:
+            mixer = self.blocks[i].mixer
+            src = getattr(mixer, "kv_from", None)
+            if src is not None:  # the layer reads the keys and values the named layer has cached (its latest run)
+                cache = of_layer[src]
+            else:
+                cache = mixer.build_cache(batch_size, self._max_seq_length, device or self.device, dtype or self.dtype)
+            of_layer[i] = cache
+            caches.append(cache)
+        self.caches = nn.ModuleList(caches)
 
     def clear_kv_cache(self) -> None:
         self.caches = None
@@ -209,20 +346,51 @@ class LayeredGPT(nn.Module):
         final residual stream (T, width) fp32 (before the final norm)."""
         if self.caches is None:
             raise TypeError("You need to call `set_kv_cache()`")
+        if self.sequential:
+            return self._forward_streams(step)
         x = seq_ops.embed(step.tokens, self.embed, self.config.embedding_scale)
         for run, layer in enumerate(self.runs):
             self.blocks[layer](x, step, self.caches[run])
         return x
 
+    def _forward_streams(self, step: StepBatch, after_layer=None) -> torch.Tensor:
+        """The sequential layers over the residual streams. Every boundary between two sublayers is one launch: the
+        write-back of the one that ran (streams mixed, output added) and the weighted read + norm of the next. The
+        last boundary reads the plain sum of the streams, which is returned. ``after_layer(run, x)``: a hook that
+        sees the streams (T, s, width) after each layer run (for tests; it costs one extra launch per layer)."""
+        eps = self.config.norm_eps
+        x = seq_ops.embed_streams(step.tokens, self.embed, self.config.embedding_scale, self.config.streams)
+        chain = [(run, sub, self.caches[run] if k == 0 else None)
+                 for run, layer in enumerate(self.runs) for k, sub in enumerate(self.blocks[layer].sublayers())]
+        first = chain[0][1]
+        got = seq_ops.streams_step(x, read=first.links.read, norm_w=first.norm_w, eps=eps,
+                                   bf16_copy=first.wants_bf16(step.T))
+        for n, (run, sub, cache) in enumerate(chain):
+            h, h16 = got if isinstance(got, tuple) else (got, None)
+            y = sub(h, h16, step, cache)
+            nxt = chain[n + 1] if n + 1 < len(chain) else None
+            if after_layer is not None and (nxt is None or nxt[0] != run):
+                seq_ops.streams_step(x, y=y, mix=sub.links.mix, out=sub.links.write)
+                after_layer(run, x)
+                y = None
+            kw = dict(y=y, mix=sub.links.mix, out=sub.links.write) if y is not None else {}
+            if nxt is None:
+                return seq_ops.streams_step(x, read=self.stream_ones, **kw)
+            got = seq_ops.streams_step(x, read=nxt[1].links.read, norm_w=nxt[1].norm_w, eps=eps,
+                                       bf16_copy=nxt[1].wants_bf16(step.T), **kw)
+        raise AssertionError("unreachable")
+
     @torch.inference_mode()
     def logits(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """Final norm and the tied output product for the given rows of the stream (int32 indices; all if None)."""
+        """Final norm and the output product (the embedding table itself, or the design's own matrix) for the given
+        rows of the stream (int32 indices; all if None)."""
         if rows is not None:
             x = seq_ops.gather_rows(x, rows)
         h = self.final_norm(x)
-        V, W = self.embed.shape
+        table = self.embed if self.head is None else self.head
+        V, W = table.shape
         out = torch.empty(h.shape[0], V, dtype=torch.float32, device=h.device)
-        return seq_ops.linear(h, self.embed, M=h.shape[0], N=V, K=W, y=out, lda=W, ldy=V)
+        return seq_ops.linear(h, table, M=h.shape[0], N=V, K=W, y=out, lda=W, ldy=V)
 
     def forward(self, idx: torch.Tensor, input_pos: Optional[torch.Tensor] = None, *,
                 last_token_only: bool = False) -> torch.Tensor:

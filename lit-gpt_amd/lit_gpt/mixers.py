@@ -13,6 +13,7 @@ dims / bases and layouts are constructor parameters; nothing is fixed to one mod
 
 from __future__ import annotations
 
+import math
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Tuple
 
@@ -21,7 +22,7 @@ import torch.nn as nn
 
 from lit_gpt import seq_ops
 from lit_gpt.config import FeedForwardSpec, MixerSpec
-from lit_gpt.model import LatentKVCache, RetentionState
+from lit_gpt.model import HeadKVCache, LatentKVCache, RetentionState, ScanState
 
 
 @dataclass
@@ -104,7 +105,8 @@ class Retention(InputReader):
     def build_cache(self, slots: int, max_seq_length: int, device, dtype) -> RetentionState:
         return RetentionState(slots, self.H, self.d, self.dv, device=device)
 
-    def forward(self, proj: torch.Tensor, step: StepBatch, cache: RetentionState, x: torch.Tensor) -> None:
+    def forward(self, proj: torch.Tensor, step: StepBatch, cache: RetentionState, x: torch.Tensor,
+                accumulate: bool = True) -> None:
         H, dv = self.H, self.dv
         o = seq_ops.retention(proj, self.off["q"], self.off["k"], self.off["v"], cache.s, self.decay, self.inv_freq,
                               step.seq_start, step.seq_slot, step.seq_pos0, H=H, d=self.d, dv=dv,
@@ -112,7 +114,7 @@ class Retention(InputReader):
         o = seq_ops.head_gate(o, proj, self.off["g"], H=H, dv=dv, unit_norm=True, eps=self.eps, act=seq_ops.ACT_SILU,
                               bf16_copy=_tiles16(step.T, self.w_o))
         W = x.shape[1]
-        seq_ops.linear(o, self.w_o, M=step.T, N=W, K=H * dv, y=x, lda=H * dv, ldy=W, accumulate=True)
+        seq_ops.linear(o, self.w_o, M=step.T, N=W, K=H * dv, y=x, lda=H * dv, ldy=W, accumulate=accumulate)
 
 
 class LatentAttention(InputReader):
@@ -147,7 +149,8 @@ class LatentAttention(InputReader):
     def build_cache(self, slots: int, max_seq_length: int, device, dtype) -> LatentKVCache:
         return LatentKVCache(slots, max_seq_length, self.r, self.dr, device=device, dtype=dtype)
 
-    def forward(self, proj: torch.Tensor, step: StepBatch, cache: LatentKVCache, x: torch.Tensor) -> None:
+    def forward(self, proj: torch.Tensor, step: StepBatch, cache: LatentKVCache, x: torch.Tensor,
+                accumulate: bool = True) -> None:
         H, d, dr, dv, r = self.H, self.d, self.dr, self.dv, self.r
         T, ld = proj.shape
         q_off = self.off["q"]
@@ -169,16 +172,134 @@ class LatentAttention(InputReader):
         att = seq_ops.head_gate(att, proj, self.off["g"], H=H, dv=dv, unit_norm=False, eps=self.eps,
                                 act=seq_ops.ACT_SIGMOID, bf16_copy=_tiles16(T, self.w_o))
         W = x.shape[1]
-        seq_ops.linear(att, self.w_o, M=T, N=W, K=H * dv, y=x, lda=H * dv, ldy=W, accumulate=True)
+        seq_ops.linear(att, self.w_o, M=T, N=W, K=H * dv, y=x, lda=H * dv, ldy=W, accumulate=accumulate)
+
+
+class DiffAttention(InputReader):
+    """Differential softmax attention with grouped key / value heads. Every query head carries two maps (the q and k
+    rows of a head are laid out [map 1 | map 2], ``dim`` each); both attend over the same values and are combined as
+    o = a1 - lambda a2 with lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + diff (one number per layer), after which the
+    head's output is divided by its root mean square and scaled by 1 - diff. Scores (q . k) * scale pass an optional
+    tanh soft cap; rotary positions on interleaved pairs (2i, 2i + 1) of the first rot.dims dims of every map; a
+    query sees the keys before it in its own chunk of ``mask_size`` positions, chunks aligned to position 0 (0: all
+    keys before it). With ``kv_from`` the layer has no key / value projections and attends over the named layer's
+    cache (rotated keys, values) with its own queries, mask and constants."""
+
+    def __init__(self, spec: MixerSpec, width: int, eps: float, w: Dict[str, torch.Tensor], device, dtype) -> None:
+        super().__init__()
+        self.H, self.G, self.d, self.dv, self.eps = spec.heads, spec.kv_heads, spec.dim, spec.vdim, eps
+        self.scale, self.cap, self.diff, self.chunk = spec.scale, spec.softcap, spec.diff, spec.mask_size
+        self.rot_dims, self.kv_from = spec.rot.dims, spec.kv_from
+        H, G, d, dv = self.H, self.G, self.d, self.dv
+        shapes = [("q", (2 * H * d, width)), ("o", (width, H * dv))]
+        if self.kv_from is None:
+            shapes += [("k", (2 * G * d, width)), ("v", (G * dv, width))]
+        for name, shape in shapes:
+            if tuple(w[name].shape) != shape:
+                raise ValueError(f"attention.{name}: shape {tuple(w[name].shape)}, expected {shape}")
+        for name in ("lq1", "lk1", "lq2", "lk2"):
+            if w[name].numel() != d:
+                raise ValueError(f"attention.{name}: {w[name].numel()} values, expected {d}")
+        self._in = [(n, w[n]) for n in (("q", "k", "v") if self.kv_from is None else ("q",))]
+        dot = lambda a, b: float((w[a].double() * w[b].double()).sum())  # noqa: E731
+        self.lam = math.exp(dot("lq1", "lk1")) - math.exp(dot("lq2", "lk2")) + self.diff
+        self.register_buffer("w_o", w["o"].to(device=device, dtype=dtype).contiguous())
+        self.register_buffer("inv_freq", torch.tensor(spec.rot.inv_freq() or [1.0], dtype=torch.float64)
+                             .to(device=device, dtype=torch.float32))
+
+    def in_parts(self):
+        return self._in
+
+    def build_cache(self, slots: int, max_seq_length: int, device, dtype) -> HeadKVCache:
+        return HeadKVCache(slots, max_seq_length, self.G, 2 * self.d, self.dv, device=device, dtype=dtype)
+
+    def forward(self, proj: torch.Tensor, step: StepBatch, cache: HeadKVCache, x: torch.Tensor,
+                accumulate: bool = True) -> None:
+        H, G, d, dv = self.H, self.G, self.d, self.dv
+        own = self.kv_from is None
+        seq_ops.diffattn_prepare(proj, self.off["q"], self.off["k"] if own else -1, self.off["v"] if own else -1,
+                                 cache.k, cache.v, self.inv_freq, step.slot, step.pos, H=H, G=G, d=d, dv=dv,
+                                 rot_dims=self.rot_dims)
+        att = seq_ops.diffattn(proj, self.off["q"], cache.k, cache.v, step.seq_start, step.seq_slot, step.seq_pos0,
+                               step.max_len or step.T, H=H, G=G, d=d, dv=dv, chunk=self.chunk, scale=self.scale,
+                               cap=self.cap, lam=self.lam, eps=self.eps, post=1.0 - self.diff,
+                               bf16_copy=_tiles16(step.T, self.w_o))
+        W = x.shape[1]
+        seq_ops.linear(att, self.w_o, M=step.T, N=W, K=H * dv, y=x, lda=H * dv, ldy=W, accumulate=accumulate)
+
+
+class SelectiveScan(InputReader):
+    """Selective state-space mixer in the Mamba-2 form. One input projection laid out [z | x | B | C | dt] (inner =
+    heads * vdim gate and value columns, groups * state columns each for B and C, one step size per head); x, B and C
+    pass a short causal per-channel convolution and silu; dt = softplus(dt + bias); per head (heads share B and C in
+    groups) S_t = exp(-exp(A_log) dt_t) S_{t-1} + dt_t B_t x_t^T, y_t = S_t^T C_t + D x_t; y is gated with silu(z),
+    divided by its root mean square in ``norm_groups`` equal parts, weighted and projected. The state (S and the
+    convolution's last taps - 1 inputs) is fp32 and lives in a cache slot."""
+
+    def __init__(self, spec: MixerSpec, width: int, eps: float, w: Dict[str, torch.Tensor], device, dtype) -> None:
+        super().__init__()
+        self.H, self.dv, self.N, self.G, self.taps = spec.heads, spec.vdim, spec.state, spec.groups, spec.conv
+        self.norm_groups, self.eps = spec.norm_groups, eps
+        inner, bc = self.H * self.dv, 2 * self.G * self.N
+        self.inner, self.channels = inner, inner + bc
+        for name, shape in (("in", (2 * inner + bc + self.H, width)), ("conv", (inner + bc, self.taps)),
+                            ("conv.b", (inner + bc,)), ("dt_bias", (self.H,)), ("A_log", (self.H,)), ("D", (self.H,)),
+                            ("norm", (inner,)), ("o", (width, inner))):
+            if tuple(w[name].shape) != shape:
+                raise ValueError(f"mamba2.{name}: shape {tuple(w[name].shape)}, expected {shape}")
+        self._in = [("in", w["in"])]
+        self.register_buffer("conv_w", w["conv"].to(device=device, dtype=dtype).contiguous())
+        self.register_buffer("conv_b", w["conv.b"].to(device=device, dtype=dtype).contiguous())
+        for name, key in (("dt_bias", "dt_bias"), ("A_log", "A_log"), ("D", "D"), ("norm_w", "norm")):
+            self.register_buffer(name, _f32(w[key], device))
+        self.register_buffer("w_o", w["o"].to(device=device, dtype=dtype).contiguous())
+
+    def in_parts(self):
+        return self._in
+
+    def build_cache(self, slots: int, max_seq_length: int, device, dtype) -> ScanState:
+        return ScanState(slots, self.H, self.N, self.dv, self.taps, self.channels, device=device)
+
+    def forward(self, proj: torch.Tensor, step: StepBatch, cache: ScanState, x: torch.Tensor,
+                accumulate: bool = True) -> None:
+        base, inner = self.off["in"], self.inner
+        tables = (step.seq_start, step.seq_slot, step.seq_pos0)
+        xbc = seq_ops.conv_silu(proj, base + inner, self.conv_w, self.conv_b, cache.conv, *tables,
+                                step.max_len or step.T)
+        y = seq_ops.ssm_scan(xbc, proj, base + inner + self.channels, self.dt_bias, self.A_log, self.D, cache.s,
+                             *tables, heads=self.H, groups=self.G, N=self.N, dv=self.dv)
+        g = seq_ops.gated_group_norm(y, proj, base, self.norm_w, groups=self.norm_groups, eps=self.eps,
+                                     bf16_copy=_tiles16(step.T, self.w_o))
+        W = x.shape[1]
+        seq_ops.linear(g, self.w_o, M=step.T, N=W, K=inner, y=x, lda=inner, ldy=W, accumulate=accumulate)
+
+
+class StreamLinks(nn.Module):
+    """The weights that tie one sublayer to a multi-stream residual: ``read`` (s,) weights of the sum the sublayer
+    reads, ``write`` (s,) weights of its output in every stream, ``mix`` (s, s) [from, to] applied to the streams
+    at the write-back. Without stored weights: all ones (one stream: the plain residual sum). fp32."""
+
+    def __init__(self, streams: int, w: Optional[Dict[str, torch.Tensor]], device) -> None:
+        super().__init__()
+        if w:
+            if w["in"].numel() != streams or w["out"].numel() != streams or tuple(w["mix"].shape) != (streams, streams):
+                raise ValueError(f"stream weights do not fit {streams} streams")
+            read, write, mix = w["in"], w["out"], w["mix"]
+        else:
+            read, write, mix = torch.ones(streams), torch.ones(streams), torch.eye(streams)
+        self.register_buffer("read", _f32(read, device))
+        self.register_buffer("write", _f32(write, device))
+        self.register_buffer("mix", _f32(mix, device))
 
 
 class GatedFeedForward(InputReader):
-    """W_down (act(W_gate h) * (W_up h)); ``act`` one of seq_ops.ACT_*."""
+    """W_down (act(W_gate h) * (W_up h)); ``act`` one of seq_ops.ACT_*. With ``clamp`` = (alpha, limit, shift) the
+    unit is g sigmoid(alpha g) (u + shift) on g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit) instead."""
 
     def __init__(self, spec: FeedForwardSpec, width: int, w: Dict[str, torch.Tensor], device, dtype,
-                 act: int = seq_ops.ACT_GELU_TANH) -> None:
+                 act: int = seq_ops.ACT_GELU_TANH, clamp: Optional[Tuple[float, float, float]] = None) -> None:
         super().__init__()
-        self.ff, self.act = spec.ff, act
+        self.ff, self.act, self.clamp = spec.ff, act, clamp
         for name, shape in (("gate", (spec.ff, width)), ("up", (spec.ff, width)), ("down", (width, spec.ff))):
             if tuple(w[name].shape) != shape:
                 raise ValueError(f"mlp.{name}: shape {tuple(w[name].shape)}, expected {shape}")
@@ -188,13 +309,18 @@ class GatedFeedForward(InputReader):
     def in_parts(self):
         return self._in
 
-    def forward(self, proj: torch.Tensor, h: torch.Tensor, x: torch.Tensor, h16=None) -> None:
+    def forward(self, proj: torch.Tensor, h: torch.Tensor, x: torch.Tensor, h16=None, accumulate: bool = True) -> None:
         # (h: the norm output, fp32 or its bf16 copy; for MFMA tiles with bf16 weights the gated product is rounded
         # where it is made)
-        a = seq_ops.glu(proj, self.off["gate"], self.off["up"], self.ff, self.act,
-                        bf16=_tiles16(proj.shape[0], self.w_down))
+        bf16 = _tiles16(proj.shape[0], self.w_down)
+        if self.clamp is not None:
+            alpha, limit, shift = self.clamp
+            a = seq_ops.glu_clamped(proj, self.off["gate"], self.off["up"], self.ff, alpha=alpha, limit=limit,
+                                    shift=shift, bf16=bf16)
+        else:
+            a = seq_ops.glu(proj, self.off["gate"], self.off["up"], self.ff, self.act, bf16=bf16)
         W = x.shape[1]
-        seq_ops.linear(a, self.w_down, M=a.shape[0], N=W, K=self.ff, y=x, lda=self.ff, ldy=W, accumulate=True)
+        seq_ops.linear(a, self.w_down, M=a.shape[0], N=W, K=self.ff, y=x, lda=self.ff, ldy=W, accumulate=accumulate)
 
 
 class SparseFeedForward(InputReader):
@@ -263,4 +389,5 @@ class TokenSide(nn.Module):
         seq_ops.token_side(x, tokens, self.table, self.col0, self.w_gate, self.w_proj, self.norm_w, self.eps)
 
 
-MIXERS = {"retention": Retention, "latent_attention": LatentAttention}
+MIXERS = {"retention": Retention, "latent_attention": LatentAttention, "attention": DiffAttention,
+          "mamba2": SelectiveScan}

@@ -671,6 +671,66 @@ class LatentKVCache(nn.Module):
         torch.nn.init.zeros_(self.kr)
 
 
+def _grown(old: torch.Tensor, slots: int) -> torch.Tensor:
+    new = torch.zeros(slots, *old.shape[1:], device=old.device, dtype=old.dtype)
+    new[: old.size(0)] = old
+    return new
+
+
+class HeadKVCache(nn.Module):
+    """Cache of an attention mixer with key / value heads of its own: per slot and position the rotated keys
+    ``k`` (kv heads, key size) and the values ``v`` (kv heads, value size), in the compute dtype. A layer that reads
+    another layer's keys and values is handed that layer's instance. A slot that is given out again needs no
+    clearing: a sequence reads only the rows it has written."""
+
+    def __init__(self, slots: int, max_seq_length: int, kv_heads: int, key_size: int, value_size: int,
+                 device: Optional[torch.device] = None, dtype: Optional[torch.dtype] = None) -> None:
+        super().__init__()
+        dtype = dtype or torch.bfloat16
+        self.register_buffer("k", torch.zeros(slots, max_seq_length, kv_heads, key_size, device=device, dtype=dtype),
+                             persistent=False)
+        self.register_buffer("v", torch.zeros(slots, max_seq_length, kv_heads, value_size, device=device, dtype=dtype),
+                             persistent=False)
+
+    @property
+    def slots(self) -> int:
+        return self.k.size(0)
+
+    def grow(self, slots: int) -> None:
+        if slots > self.slots:
+            self.k, self.v = _grown(self.k, slots), _grown(self.v, slots)
+
+    def reset_parameters(self) -> None:
+        torch.nn.init.zeros_(self.k)
+        torch.nn.init.zeros_(self.v)
+
+
+class ScanState(nn.Module):
+    """Per-slot state of a selective state-space mixer, fp32: the recurrent state ``s`` (heads, state size, value
+    dim) and the short convolution's last inputs ``conv`` (taps - 1, channels), oldest first. The kernels take zeros
+    for a sequence that starts at position 0, so a slot that is given out again needs no clearing."""
+
+    def __init__(self, slots: int, heads: int, state: int, vdim: int, taps: int, channels: int,
+                 device: Optional[torch.device] = None) -> None:
+        super().__init__()
+        self.register_buffer("s", torch.zeros(slots, heads, state, vdim, device=device, dtype=torch.float32),
+                             persistent=False)
+        self.register_buffer("conv", torch.zeros(slots, max(1, taps - 1), channels, device=device, dtype=torch.float32),
+                             persistent=False)
+
+    @property
+    def slots(self) -> int:
+        return self.s.size(0)
+
+    def grow(self, slots: int) -> None:
+        if slots > self.slots:
+            self.s, self.conv = _grown(self.s, slots), _grown(self.conv, slots)
+
+    def reset_parameters(self) -> None:
+        torch.nn.init.zeros_(self.s)
+        torch.nn.init.zeros_(self.conv)
+
+
 def build_rope_cache(seq_len: int, n_elem: int, device: Optional[torch.device] = None, base: int = 10000,
                      condense_ratio: int = 1) -> Tuple[torch.Tensor, torch.Tensor]:
     """cos/sin tables (seq_len, n_elem) in fp32 (model.py:746-764).

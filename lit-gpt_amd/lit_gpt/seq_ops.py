@@ -47,6 +47,15 @@ SIGNATURES = {
     "lgs_moe_sort": [_P, _I, _I, _I, _P, _P, _P, _P, _P],
     "lgs_moe_combine": [_P, _P, _P, _P, _L, _I, _I, _I, _P],
     "lgs_token_side": [_P, _P, _P, _I, _L, _I, _P, _P, _P, _I, _I, _I, _I, _F, _P],
+    "lgs_embed_streams": [_P, _P, _I, _F, _P, _I, _I, _I, _I, _P],
+    "lgs_streams_step": [_P, _P, _P, _P, _P, _P, _P, _P, _F, _I, _I, _I, _P],
+    "lgs_diffattn_prepare": [_P, _L, _I, _I, _I, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
+    "lgs_diffattn": [_P, _L, _P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _F, _F, _F, _F,
+                     _F, _P],
+    "lgs_conv_silu": [_P, _L, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
+    "lgs_ssm_scan": [_P, _L, _P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
+    "lgs_gated_group_norm": [_P, _P, _L, _P, _F, _P, _P, _I, _I, _I, _P],
+    "lgs_glu_clamped": [_P, _P, _L, _P, _I, _I, _I, _F, _F, _F, _P],
 }
 _RESTYPES = {"lgs_last_error_string": ctypes.c_char_p}
 
@@ -354,3 +363,157 @@ def token_side(x: torch.Tensor, tokens: torch.Tensor, table: torch.Tensor, col0:
                                          _wf32(table, "table"), ld, col0, _dev(gate_w, "gate_w"),
                                          _dev(proj_w, "proj_w"), _dev(norm_w, "norm_w", F32), T, W, dim, V,
                                          float(eps), _stream()))
+
+
+def embed_streams(tokens: torch.Tensor, table: torch.Tensor, scale: float, streams: int) -> torch.Tensor:
+    """(T, streams, W) fp32: every stream starts as the scaled embedding row."""
+    T, (V, W) = tokens.numel(), table.shape
+    x = torch.empty(T, streams, W, dtype=F32, device=tokens.device)
+    _check(load_library().lgs_embed_streams(_dev(tokens, "tokens", I32), _dev(table, "table"), _wf32(table, "table"),
+                                            float(scale), x.data_ptr(), T, W, V, streams, _stream()))
+    return x
+
+
+def streams_step(x: torch.Tensor, *, y: Optional[torch.Tensor] = None, mix: Optional[torch.Tensor] = None,
+                 out: Optional[torch.Tensor] = None, read: Optional[torch.Tensor] = None,
+                 norm_w: Optional[torch.Tensor] = None, eps: float = 0.0, bf16_copy: bool = False):
+    """One sublayer boundary of a multi-stream residual x (T, s, W), in place: with ``y`` (T, W) the write-back
+    x_j <- sum_i mix[i, j] x_i + out[j] y; then with ``read`` (s,) the next sublayer's input
+    h = rmsnorm(sum_j read[j] x_j) * norm_w (no ``norm_w``: the weighted sum itself). Returns None without a read,
+    else h, or (h, h_bf16) with ``bf16_copy``."""
+    T, s, W = x.shape
+    if y is not None and (y.shape != (T, W) or mix is None or out is None or mix.numel() != s * s or out.numel() != s):
+        raise ValueError("streams_step: write-back shapes")
+    if read is not None and (read.numel() != s or (norm_w is not None and norm_w.numel() != W)):
+        raise ValueError("streams_step: read shapes")
+    h = torch.empty(T, W, dtype=F32, device=x.device) if read is not None else None
+    h16 = torch.empty(T, W, dtype=torch.bfloat16, device=x.device) if read is not None and bf16_copy else None
+    _check(load_library().lgs_streams_step(_dev(x, "x", F32), _opt(y, "y", F32), _opt(mix, "mix", F32),
+                                           _opt(out, "out", F32), _opt(read, "read", F32), _opt(norm_w, "norm_w", F32),
+                                           _opt(h, "h", F32), _opt(h16, "h_bf16", torch.bfloat16), float(eps), T, W, s,
+                                           _stream()))
+    if read is None:
+        return None
+    return (h, h16) if bf16_copy else h
+
+
+def diffattn_prepare(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, cache_k: Optional[torch.Tensor],
+                     cache_v: Optional[torch.Tensor], inv_freq: Optional[torch.Tensor], slot: torch.Tensor,
+                     pos: torch.Tensor, *, H: int, G: int, d: int, dv: int, rot_dims: int) -> None:
+    """Rotates the query maps of ``proj`` in place; with key / value columns (``k_off`` >= 0) the rotated keys and
+    the values go to the cache rows (slot, position). cache_k (slots, S, G, 2 d), cache_v (slots, S, G, dv)."""
+    T, ld = proj.shape
+    S = 1
+    if k_off >= 0:
+        slots, S = cache_k.shape[:2]
+        if tuple(cache_k.shape) != (slots, S, G, 2 * d) or tuple(cache_v.shape) != (slots, S, G, dv) or \
+                cache_k.dtype != cache_v.dtype:
+            raise ValueError("diffattn_prepare: cache shapes")
+    if slot.numel() != T or pos.numel() != T:
+        raise ValueError("diffattn_prepare: one slot and position per row")
+    f32 = _wf32(cache_k, "cache_k") if k_off >= 0 else 1
+    _check(load_library().lgs_diffattn_prepare(_dev(proj, "proj", F32), ld, q_off, k_off, v_off,
+                                               _dev(cache_k, "cache_k") if k_off >= 0 else None,
+                                               _dev(cache_v, "cache_v") if k_off >= 0 else None, f32,
+                                               _opt(inv_freq, "inv_freq", F32), _dev(slot, "slot", I32),
+                                               _dev(pos, "pos", I32), T, H, G, d, dv, rot_dims, S, _stream()))
+
+
+def diffattn(proj: torch.Tensor, q_off: int, cache_k: torch.Tensor, cache_v: torch.Tensor, seq_start: torch.Tensor,
+             seq_slot: torch.Tensor, seq_pos0: torch.Tensor, max_len: int, *, H: int, G: int, d: int, dv: int,
+             chunk: int, scale: float, cap: float, lam: float, eps: float, post: float, bf16_copy: bool = False,
+             splits: Optional[int] = None) -> torch.Tensor:
+    """Differential attention of every row of a packed batch over its sequence's cached keys and values; the
+    rotated queries are the 2 H d columns of ``proj`` at ``q_off``. Returns (T, H dv) fp32, or with ``bf16_copy``
+    its rounding to bf16 (the out-projection's MFMA operand). ``splits``: workgroups per (token, head) when every
+    sequence brings one token (default: enough to fill the chip, at least 128 keys each)."""
+    T, ld = proj.shape
+    B = seq_slot.numel()
+    slots, S = cache_k.shape[:2]
+    if tuple(cache_k.shape) != (slots, S, G, 2 * d) or tuple(cache_v.shape) != (slots, S, G, dv):
+        raise ValueError("diffattn: cache shapes")
+    if seq_start.numel() != B + 1 or q_off + 2 * H * d > ld or not 1 <= max_len <= T:
+        raise ValueError("diffattn: step table / query columns")
+    out = torch.empty(T, H * dv, dtype=F32, device=proj.device)
+    out16 = torch.empty(T, H * dv, dtype=torch.bfloat16, device=proj.device) if bf16_copy else None
+    if max_len > 1:
+        splits = 1
+    elif splits is None:
+        span = min(S, chunk) if chunk > 0 else S
+        splits = max(1, min(64, 512 // max(1, B * H), (span + 127) // 128))
+    part = torch.empty(T * H * splits * (4 + 2 * dv), dtype=F32, device=proj.device) if splits > 1 else None
+    _check(load_library().lgs_diffattn(_dev(proj, "proj", F32) + 4 * q_off, ld, _dev(cache_k, "cache_k"),
+                                       _dev(cache_v, "cache_v"), _wf32(cache_k, "cache_k"),
+                                       _dev(seq_start, "seq_start", I32), _dev(seq_slot, "seq_slot", I32),
+                                       _dev(seq_pos0, "seq_pos0", I32), out.data_ptr(),
+                                       _opt(out16, "out_bf16", torch.bfloat16), _opt(part, "part", F32), splits, B,
+                                       int(max_len), H, G, d, dv, S, int(chunk), float(scale), float(cap), float(lam),
+                                       float(eps), float(post), _stream()))
+    return out16 if bf16_copy else out
+
+
+def conv_silu(proj: torch.Tensor, off: int, weight: torch.Tensor, bias: torch.Tensor, state: torch.Tensor,
+              seq_start: torch.Tensor, seq_slot: torch.Tensor, seq_pos0: torch.Tensor, max_len: int) -> torch.Tensor:
+    """silu(causal per-channel convolution + bias) of the C columns of ``proj`` at ``off`` over a packed batch;
+    weight (C, taps), last column the current token's. state (slots, taps - 1, C) fp32 carries every sequence's last
+    inputs from step to step. Returns (T, C) fp32."""
+    T, ld = proj.shape
+    C, taps = weight.shape
+    B = seq_slot.numel()
+    if off + C > ld or bias.numel() != C or tuple(state.shape[1:]) != (taps - 1, C) or weight.dtype != bias.dtype:
+        raise ValueError("conv_silu: shapes")
+    out = torch.empty(T, C, dtype=F32, device=proj.device)
+    _check(load_library().lgs_conv_silu(_dev(proj, "proj", F32) + 4 * off, ld, _dev(weight, "weight"),
+                                        _dev(bias, "bias"), _wf32(weight, "weight"), _dev(state, "state", F32),
+                                        _dev(seq_start, "seq_start", I32), _dev(seq_slot, "seq_slot", I32),
+                                        _dev(seq_pos0, "seq_pos0", I32), out.data_ptr(), B, int(max_len), C, taps,
+                                        _stream()))
+    return out
+
+
+def ssm_scan(xbc: torch.Tensor, proj: torch.Tensor, dt_off: int, dt_bias: torch.Tensor, A_log: torch.Tensor,
+             D: torch.Tensor, state: torch.Tensor, seq_start: torch.Tensor, seq_slot: torch.Tensor,
+             seq_pos0: torch.Tensor, *, heads: int, groups: int, N: int, dv: int) -> torch.Tensor:
+    """The selective scan over a packed batch: xbc (T, heads dv + 2 groups N) after the convolution, raw step sizes
+    in the ``heads`` columns of ``proj`` at ``dt_off``; state (slots, heads, N, dv) fp32. Returns y (T, heads dv)."""
+    T, ldx = xbc.shape
+    B = seq_slot.numel()
+    if ldx != heads * dv + 2 * groups * N or tuple(state.shape[1:]) != (heads, N, dv) or proj.shape[0] != T:
+        raise ValueError("ssm_scan: shapes")
+    if dt_off + heads > proj.shape[1] or min(dt_bias.numel(), A_log.numel(), D.numel()) != heads:
+        raise ValueError("ssm_scan: per-head parameters")
+    y = torch.empty(T, heads * dv, dtype=F32, device=xbc.device)
+    _check(load_library().lgs_ssm_scan(_dev(xbc, "xbc", F32), ldx, _dev(proj, "proj", F32) + 4 * dt_off,
+                                       proj.shape[1], _dev(dt_bias, "dt_bias", F32), _dev(A_log, "A_log", F32),
+                                       _dev(D, "D", F32), _dev(state, "state", F32), _dev(seq_start, "seq_start", I32),
+                                       _dev(seq_slot, "seq_slot", I32), _dev(seq_pos0, "seq_pos0", I32), y.data_ptr(),
+                                       B, heads, groups, N, dv, _stream()))
+    return y
+
+
+def gated_group_norm(y: torch.Tensor, proj: torch.Tensor, z_off: int, weight: torch.Tensor, *, groups: int,
+                     eps: float, bf16_copy: bool = False) -> torch.Tensor:
+    """unit_rms_per_group(y * silu(z)) * weight with z the columns of ``proj`` at ``z_off``; (T, inner) fp32 or, with
+    ``bf16_copy``, its rounding to bf16."""
+    T, inner = y.shape
+    if z_off + inner > proj.shape[1] or weight.numel() != inner or inner % groups:
+        raise ValueError("gated_group_norm: shapes")
+    out = torch.empty(T, inner, dtype=F32, device=y.device)
+    out16 = torch.empty(T, inner, dtype=torch.bfloat16, device=y.device) if bf16_copy else None
+    _check(load_library().lgs_gated_group_norm(_dev(y, "y", F32), _dev(proj, "proj", F32) + 4 * z_off, proj.shape[1],
+                                               _dev(weight, "weight", F32), float(eps), out.data_ptr(),
+                                               _opt(out16, "out_bf16", torch.bfloat16), T, inner, groups, _stream()))
+    return out16 if bf16_copy else out
+
+
+def glu_clamped(proj: torch.Tensor, a_off: int, b_off: int, n: int, *, alpha: float, limit: float, shift: float,
+                bf16: bool = False) -> torch.Tensor:
+    """g sigmoid(alpha g) (u + shift) with g = min(proj[:, a_off:], limit), u = clamp(proj[:, b_off:], +-limit)."""
+    T, ld = proj.shape
+    if max(a_off, b_off) + n > ld:
+        raise ValueError("glu_clamped: columns outside the row")
+    out = torch.empty(T, n, dtype=torch.bfloat16 if bf16 else F32, device=proj.device)
+    base = _dev(proj, "proj", F32)
+    _check(load_library().lgs_glu_clamped(base + 4 * a_off, base + 4 * b_off, ld, out.data_ptr(), int(bf16), T, n,
+                                          float(alpha), float(limit), float(shift), _stream()))
+    return out
