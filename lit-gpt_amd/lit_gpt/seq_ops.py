@@ -460,7 +460,7 @@ def conv_silu(proj: torch.Tensor, off: int, weight: torch.Tensor, bias: torch.Te
     T, ld = proj.shape
     C, taps = weight.shape
     B = seq_slot.numel()
-    if off + C > ld or bias.numel() != C or tuple(state.shape[1:]) != (taps - 1, C) or weight.dtype != bias.dtype:
+    if off + C > ld or bias.numel() != C or tuple(state.shape[1:]) != (max(1, taps - 1), C) or weight.dtype != bias.dtype:
         raise ValueError("conv_silu: shapes")
     out = torch.empty(T, C, dtype=F32, device=proj.device)
     _check(load_library().lgs_conv_silu(_dev(proj, "proj", F32) + 4 * off, ld, _dev(weight, "weight"),

@@ -99,11 +99,10 @@ def diff_attention(h: torch.Tensor, w: Dict[str, torch.Tensor], m: dict, eps: fl
             maps = []
             for a in range(2):
                 qt = rope_interleaved(q[t, hd, a], t, rot["dims"], rot["base"])
-                s = torch.stack([(qt * keys[j, g, a]).sum() for j in js]) * float(m["scale"])
+                s = (keys[js, g, a] @ qt) * float(m["scale"])
                 if cap:
                     s = float(cap) * torch.tanh(s / float(cap))
-                p = torch.softmax(s, 0)
-                maps.append(sum(p[n] * vals[j, g] for n, j in enumerate(js)))
+                maps.append(torch.softmax(s, 0) @ vals[js, g])
             o = maps[0] - lam * maps[1]
             out[t, hd] = rms_unit(o, eps) * (1.0 - float(m["diff"]))
     return out.reshape(T, H * dv) @ w["o"].T
