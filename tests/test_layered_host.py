@@ -174,3 +174,87 @@ def test_oracle_is_causal_and_loops_share_weights():
         torch.sin(torch.tensor(1.0, dtype=torch.float64)).item())
     assert ob.rope_interleaved(torch.tensor([1.0, 0, 0, 0], dtype=torch.float64), 1, 4, 100.0)[1] == pytest.approx(
         torch.sin(torch.tensor(1.0, dtype=torch.float64)).item())
+
+
+# ------------------------------------------------------------------------------------------------ Rigulorn
+def _rig_cfg():
+    att = {"heads": 4, "kv_heads": 2, "dim": 6, "vdim": 10, "diff": 0.3, "softcap": 9.0, "scale": 0.35,
+           "mask": {"size": 5}, "rot": {"dims": 4, "base": 300.0}}
+    return {
+        "architecture": "Rigulorn", "vocab": 23, "width": 16, "norm": {"eps": 1e-5}, "embedding": {"scale": 4.0},
+        "streams": 2,
+        "layers": [
+            {"type": "mamba2", "mlp": None,
+             "mixer": {"heads": 4, "vdim": 3, "state": 5, "groups": 2, "norm_groups": 3, "conv": 4}},
+            {"type": "attention", "mlp": {"kind": "dense", "ff": 14, "limit": 1.25}, "mixer": dict(att)},
+            {"type": "attention", "mlp": None, "mixer": dict(att, kv_from=1, mask={"size": 3})},
+        ]}
+
+
+def test_rigulorn_config_and_tensor_names():
+    from lit_gpt.config import LayeredConfig, model_class
+    from lit_gpt.layered import LayeredGPT
+
+    c = LayeredConfig.from_dict(_rig_cfg())
+    assert model_class(c) is LayeredGPT
+    assert (c.streams, c.stream_weights, c.design.block, c.design.tied_head) == (2, True, "sequential", False)
+    s, a, b = (l.mixer for l in c.layers)
+    assert (s.kind, s.heads, s.vdim, s.state, s.groups, s.norm_groups, s.conv) == ("mamba2", 4, 3, 5, 2, 3, 4)
+    assert (a.kv_heads, a.diff, a.softcap, a.mask_size, a.scale, a.rot.dims, a.kv_from) == (2, 0.3, 9.0, 5, 0.35, 4, None)
+    assert (b.kv_from, b.mask_size) == (1, 3) and c.layers[1].mlp.limit == 1.25
+    shapes = LayeredGPT.tensor_shapes(c)
+    assert shapes["head"] == (23, 16) and shapes["l0.mix.in"] == (2 * 12 + 2 * 2 * 5 + 4, 16)
+    assert shapes["l0.mix.conv"] == (12 + 20, 4) and shapes["l0.hc1.mix"] == (2, 2) and "l0.hc2.in" not in shapes
+    assert shapes["l1.mix.q"] == (48, 16) and shapes["l1.mix.k"] == (24, 16) and shapes["l1.mix.v"] == (20, 16)
+    assert "l2.mix.k" not in shapes and "l2.mix.v" not in shapes and "l2.norm2" not in shapes
+    assert shapes["l1.norm2"] == (16,) and shapes["l1.mix.lq2"] == (6,)
+    w = LayeredGPT.random_weights(c)
+    assert set(w) == set(shapes) and all(tuple(w[k].shape) == shapes[k] for k in shapes)
+    plain = dict(_rig_cfg())
+    del plain["streams"]
+    p = LayeredConfig.from_dict(plain)
+    assert p.streams == 1 and not p.stream_weights and "l0.hc1.in" not in LayeredGPT.tensor_shapes(p)
+
+
+@pytest.mark.parametrize("edit", [
+    lambda c: c["layers"][2]["mixer"].update(kv_from=0),  # not an attention layer
+    lambda c: c["layers"][2]["mixer"].update(kv_from=2),  # itself
+    lambda c: c["layers"][2]["mixer"].update(kv_heads=4),  # other key heads than its source
+    lambda c: c["layers"][1]["mixer"].update(kv_heads=3),
+    lambda c: c["layers"][0]["mixer"].update(groups=3),
+    lambda c: c["layers"][0]["mixer"].update(norm_groups=5),
+    lambda c: c["layers"][1]["mixer"]["rot"].update(dims=8),
+    lambda c: c.update(streams=9),
+])
+def test_rigulorn_config_rejects_what_does_not_fit(edit):
+    from lit_gpt.config import LayeredConfig
+
+    c = _rig_cfg()
+    edit(c)
+    with pytest.raises(ValueError):
+        LayeredConfig.from_dict(c)
+
+
+def test_rigulorn_plain_implementation_is_causal_and_chunked():
+    from lit_gpt.config import LayeredConfig
+    from lit_gpt.layered import LayeredGPT
+    from oracle import rigulorn as orc
+
+    cfg = _rig_cfg()
+    w = LayeredGPT.random_weights(LayeredConfig.from_dict(cfg), seed=3)
+    toks = [3, 7, 1, 0, 22, 5, 9, 9, 4, 13, 2, 8]
+    full = orc.forward(cfg, w, toks)
+    assert torch.allclose(orc.forward(cfg, w, toks[:7]), full[:7], atol=1e-10)
+    # attention alone: a token before the query's chunk cannot reach it (values are per-token maps of the embedding)
+    only = dict(cfg, layers=[dict(cfg["layers"][1], mlp=None)])
+    w1 = {k: v for k, v in LayeredGPT.random_weights(LayeredConfig.from_dict(only), seed=4).items()}
+    a = orc.forward(only, w1, toks)
+    other = list(toks)
+    other[4] = 11  # the last position of the first chunk of 5
+    b = orc.forward(only, w1, other)
+    assert torch.allclose(a[5:], b[5:], atol=1e-12) and not torch.allclose(a[4], b[4], atol=1e-6)
+    assert orc.visible(9, 5, {"size": 5}) and not orc.visible(9, 4, {"size": 5}) and not orc.visible(4, 5, None)
+    # the convolution's last column is the current token's
+    u = torch.arange(6.0, dtype=torch.float64).view(6, 1)
+    got = orc.causal_conv(u, torch.tensor([[0.0, 0.0, 1.0]], dtype=torch.float64), torch.zeros(1, dtype=torch.float64))
+    assert torch.equal(got, u)
