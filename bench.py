@@ -494,12 +494,128 @@ def layered_bench(args) -> None:
         print(json.dumps(line), flush=True)
 
 
+def hybrid_bench(args) -> None:
+    """``--hybrid``: prefill and decode throughput of the Rigulorn design (state-space and differential-attention
+    layers over four residual streams, random bf16 weights) at sizes that resemble a real model's layers, beside the
+    closest existing model — a Llama-family stack in bf16 — at equal width, depth, query-head count and feed-forward
+    size. One JSON line per size. Prefill: one 2048-token prompt, warm, median of 3. Decode: captured greedy steps at
+    context 2048 (both models through their HIP-graph executors), and for the hybrid also a batch of 8 sequences.
+    ``hbm_frac``: algorithmic bytes of a decode step over 8 TB/s."""
+    from generate.base import build_model
+    from generate.batch import BatchEngine
+    from lit_gpt import Config, ops
+    from lit_gpt.config import LayeredConfig
+    from lit_gpt.layered import LayeredGPT
+    from lit_gpt.runtime import DecodeGraph
+
+    dev = torch.device("cuda", 0)
+    T, steps, L, V = args.prompt_len, args.steps, 4, 32000
+    sizes = {"w2048": (2048, 5632), "w4096": (4096, 11008)}
+
+    def timed(fn, reps=3):
+        out = []
+        for _ in range(reps):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            fn()
+            torch.cuda.synchronize()
+            out.append(time.perf_counter() - t0)
+        return sorted(out)[len(out) // 2]
+
+    for name, (W, ff) in sizes.items():
+        if args.hybrid not in ("all", name):
+            continue
+        H = W // 128
+        att = {"heads": H, "kv_heads": H // 4, "dim": 64, "vdim": 128, "diff": 0.5, "softcap": 30.0, "scale": 0.125,
+               "mask": {"size": 1024}, "rot": {"dims": 64, "base": 1e4}}
+        ssm = {"type": "mamba2", "mixer": {"heads": 2 * W // 64, "vdim": 64, "state": 128, "groups": 8, "norm_groups": 8,
+                                           "conv": 4}}
+        mlp = {"kind": "dense", "ff": ff, "limit": 7.0}
+        cfg = LayeredConfig.from_dict({
+            "architecture": "Rigulorn", "vocab": V, "width": W, "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0},
+            "streams": 4,
+            "layers": [dict(ssm, mlp=mlp), {"type": "attention", "mixer": att, "mlp": mlp}, dict(ssm, mlp=mlp),
+                       {"type": "attention", "mixer": dict(att, kv_from=1), "mlp": mlp}]})
+        line = {"bench": "hybrid", "size": name, "width": W, "ff": ff, "layers": L, "prompt_len": T, "steps": steps,
+                "dtype": "bf16", "data": "synthetic"}
+        model = LayeredGPT(cfg, LayeredGPT.random_weights(cfg, seed=1), device=dev, dtype=torch.bfloat16)
+        g = torch.Generator().manual_seed(1234)
+        res = {}
+        for B in (1, 8):
+            eng = BatchEngine(model, max_seq_length=T + steps + args.warmup + 8, slots=B)
+            prompts = [torch.randint(0, V, (T,), generator=g).tolist() for _ in range(B)]
+            ids = list(range(B))
+            with torch.inference_mode():
+                def prefill():
+                    for r in list(eng.live):
+                        eng.step([], end=[r])
+                    return eng.step([(i, prompts[i], [T - 1]) for i in ids])
+                prefill()
+                res[f"prefill_tok_s_b{B}"] = round(B * T / timed(prefill))
+                lg = prefill()
+                first = [int(torch.argmax(lg[i])) for i in ids]
+                graph = eng.decode_graph(ids, first)
+                graph.step()
+                for _ in range(args.warmup):
+                    graph.step()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(steps):
+                    graph.step()
+                torch.cuda.synchronize()
+                dt = (time.perf_counter() - t0) / steps
+            res[f"decode_tok_s_b{B}"] = round(B / dt, 1)
+            res[f"decode_ms_step_b{B}"] = round(dt * 1e3, 4)
+            del eng, graph
+            model.clear_kv_cache()
+        # algorithmic traffic of a decode step (B = 1): every matrix once in bf16, the visible key / value rows of the
+        # attention layers (bf16; half a chunk on average), the recurrent states (fp32, read and written)
+        mat = sum(sub.w_in.numel() + (sub.module.w_o if k == 0 else sub.module.w_down).numel()
+                  for blk in model.blocks for k, sub in enumerate(blk.sublayers()))
+        kv = 2 * 512 * (H // 4) * (128 + 128) * 2
+        state = 2 * 2 * (2 * W // 64) * 128 * 64 * 4
+        res["hbm_frac_decode_b1"] = round((2 * (mat + V * W) + kv + state) / (res["decode_ms_step_b1"] * 1e-3)
+                                          / (HBM_PEAK_GBS * 1e9), 3)
+        line["hybrid"] = res
+        del model
+        torch.cuda.empty_cache()
+        lcfg = Config.from_name("Llama-2-7b-hf", n_layer=L, n_embd=W, n_head=H, intermediate_size=ff, vocab_size=V,
+                                padding_multiple=64, block_size=T + steps + 4)
+        lm = build_model(lcfg, quantize=None, device=dev, max_seq_length=T + steps + 4, prefill_rows=T)
+        prompt = torch.randint(0, V, (T,), generator=torch.Generator().manual_seed(1234), dtype=torch.int32).to(dev)
+        with torch.inference_mode():
+            def lprefill():
+                return lm(prompt.view(1, -1), torch.arange(T, device=dev), last_token_only=True)
+            lprefill()
+            res = {"prefill_tok_s_b1": round(T / timed(lprefill))}
+            first = ops.argmax(lprefill().reshape(-1)).to(torch.int32)
+            dg = DecodeGraph(lm, first, T, chunk=1)
+            for _ in range(args.warmup):
+                dg.step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                dg.step()
+            torch.cuda.synchronize()
+            dt = (time.perf_counter() - t0) / steps
+        res["decode_tok_s_b1"], res["decode_ms_step_b1"] = round(1 / dt, 1), round(dt * 1e3, 4)
+        res["hbm_frac_decode_b1"] = round(algorithmic_bytes_per_token(lcfg, T + steps / 2, dense=True) / dt
+                                          / (HBM_PEAK_GBS * 1e9), 3)
+        line["llama_bf16"] = res
+        del lm, dg
+        torch.cuda.empty_cache()
+        print(json.dumps(line), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--layered", nargs="?", const="all", default=None, choices=("all", "w2048", "w4096"),
                     help="instead of the headline run: the layered design beside a Llama-family stack of equal size "
                          "(prefill and decode throughput, one JSON line per size)")
+    ap.add_argument("--hybrid", nargs="?", const="all", default=None, choices=("all", "w2048", "w4096"),
+                    help="instead of the headline run: the Rigulorn design (state-space and differential-attention "
+                         "layers over several residual streams) beside a Llama-family stack of equal size")
     # defaults: the eager capture step (p = 2048) + 14 warm-up + 240 timed steps = the 255 decode steps of
     # SURVEY §8d (p = 2048 ... 2302)
     ap.add_argument("--steps", type=int, default=240)
@@ -521,6 +637,8 @@ def main():
         return pmc_child(args.pmc_pos)
     if args.layered:
         return layered_bench(args)
+    if args.hybrid:
+        return hybrid_bench(args)
     traffic = {k: (None, "skipped") for k in ("gemv", "attention")}
     under_profiler = any(k.startswith(("ROCPROF", "ROCP_")) for k in os.environ)
     headline = args.model == MODEL and args.quantize == "int4-g128"

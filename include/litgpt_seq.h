@@ -148,10 +148,14 @@ int lgs_conv_silu(const float* u, long ld, const void* w, const void* bias, int 
                   int taps, lgs_stream_t stream);
 /* Per sequence and head: dt = softplus(dt_raw + dt_bias), S <- exp(-exp(A_log) dt) S + dt B x^T, y = S^T C + D x.
  * xbc rows hold x [heads][dv] | B [groups][N] | C [groups][N]; head h reads group h / (heads / groups).
- * state [slots][heads][N][dv] fp32 is read unless the sequence starts at position 0, and written back. N <= 256. */
+ * state [slots][heads][N][dv] fp32 is read unless the sequence starts at position 0, and written back. N <= 256.
+ * With a workspace (ws: B max_chunks heads N dv floats, wdec: B max_chunks heads floats; max_chunks = 64-token chunks
+ * of the longest sequence; N <= 128) the prompt form runs: chunks as fp32 matrix products side by side, a short
+ * carry over the chunks, then the outputs. Without (ws NULL) the tokens are walked one by one. */
 int lgs_ssm_scan(const float* xbc, long ldx, const float* dt, long ldd, const float* dt_bias, const float* A_log,
                  const float* D, float* state, const int* seq_start, const int* seq_slot, const int* seq_pos0,
-                 float* y, int B, int heads, int groups, int N, int dv, lgs_stream_t stream);
+                 float* y, int B, int heads, int groups, int N, int dv, float* ws, float* wdec, int max_chunks,
+                 lgs_stream_t stream);
 /* out = v / sqrt(mean over the group of v^2 + eps) * w, v = y * silu(z); `groups` equal parts of `inner` columns */
 int lgs_gated_group_norm(const float* y, const float* z, long ldz, const float* w, float eps, float* out,
                          void* out_bf16, int T, int inner, int groups, lgs_stream_t stream);

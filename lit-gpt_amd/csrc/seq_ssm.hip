@@ -5,7 +5,8 @@
 //                        of a step that continues a sequence and rewritten at its end
 //   lgs_ssm_scan         per head: dt = softplus(raw + bias), a = exp(-exp(A_log) dt),
 //                        S <- a S + dt B x^T (S is N x dv, fp32, one per cache slot), y = S^T C + D x;
-//                        heads share B and C in groups
+//                        heads share B and C in groups. Token by token (decode, short portions), or for prompts
+//                        in chunks of 64 tokens as fp32 matrix products with the chunks side by side
 //   lgs_gated_group_norm out = unit_rms_per_group(y * silu(z)) * w: the gate comes before the norm
 #include "seq_common.h"
 
@@ -155,6 +156,192 @@ __global__ void __launch_bounds__(256) ssm_scan_kernel(ScanArgs p) {
   }
 }
 
+// The prompt form of the scan: chunks of 64 tokens as fp32 matrix products (v_mfma_f32_16x16x4_f32), all chunks of
+// all sequences side by side. With l_i the running sum of log a over the chunk's tokens up to i, S0 the state at the
+// chunk's start and n its token count:
+//   y_i = exp(l_i) C_i^T S0 + sum_{j <= i} exp(l_i - l_j) dt_j (C_i . B_j) x_j + D x_i
+//   S'  = exp(l_{n-1}) S0 + sum_j exp(l_{n-1} - l_j) dt_j B_j x_j^T
+// MODE 1, grid (B * max_chunks, heads, ceil(dv / 64)): the second term of S' of every chunk -> workspace, the chunk's
+// whole decay -> wdec. ssd_carry_kernel turns these into the state at each chunk's start (an elementwise recurrence
+// over the chunks, which also leaves the final state in the slot). MODE 2: the outputs of every chunk.
+// LDS (floats): C, B [64][NP + 2], x [64][80], scores [64][66], l, dt, weights [64] each; N <= 128.
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+constexpr int kSC = 64, kXS = 80, kGS = 66;
+
+struct SsdArgs {
+  const float* xbc;
+  long ldx;
+  const float* dt;
+  long ldd;
+  const float *dt_bias, *A_log, *D;
+  float* state;
+  const int *seq_start, *seq_slot, *seq_pos0;
+  float* y;
+  float* ws;    // [B * max_chunks][heads][N][dv]
+  float* wdec;  // [B * max_chunks][heads]
+  int heads, groups, N, dv, max_chunks;
+};
+
+template <int MODE>
+__global__ void __launch_bounds__(256) ssd_chunk_kernel(SsdArgs p) {
+  extern __shared__ float lds[];
+  const int b = blockIdx.x / p.max_chunks, cidx = blockIdx.x % p.max_chunks;
+  const int h = blockIdx.y, col0 = blockIdx.z * 64;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int t0 = p.seq_start[b], t1 = p.seq_start[b + 1];
+  const int tc = t0 + cidx * kSC;
+  if (tc >= t1) return;
+  const int n = min(kSC, t1 - tc);
+  const int N = p.N, dv = p.dv, H = p.heads, inner = H * dv;
+  const int g = h / (H / p.groups);
+  const int NP = (N + 15) / 16 * 16, NS = NP + 2;
+  float* Cs = lds;
+  float* Bs = Cs + kSC * NS;
+  float* Xs = Bs + kSC * NS;
+  float* Gs = Xs + kSC * kXS;
+  float* la = Gs + kSC * kGS;
+  float* dts = la + kSC;
+  float* wgt = dts + kSC;
+  if (wave == 0) {
+    float d = 0.0f, l = 0.0f;
+    if (lane < n) {
+      d = softplus_f(p.dt[(size_t)(tc + lane) * p.ldd + h] + p.dt_bias[h]);
+      l = -expf(p.A_log[h]) * d;
+    }
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const float v = __shfl_up(l, o);
+      if (lane >= o) l += v;
+    }
+    la[lane] = l;
+    dts[lane] = d;
+  }
+  for (int i = tid; i < kSC * NP; i += 256) {
+    const int row = i / NP, k = i - row * NP;
+    const bool in = row < n && k < N;
+    const size_t at = (size_t)(tc + row) * p.ldx + inner + (size_t)g * N + k;
+    Bs[row * NS + k] = in ? p.xbc[at] : 0.0f;
+    if (MODE == 2) Cs[row * NS + k] = in ? p.xbc[at + (size_t)p.groups * N] : 0.0f;
+  }
+  for (int i = tid; i < kSC * 64; i += 256) {
+    const int row = i >> 6, c = i & 63;
+    Xs[row * kXS + c] = (row < n && col0 + c < dv) ? p.xbc[(size_t)(tc + row) * p.ldx + (size_t)h * dv + col0 + c] : 0.0f;
+  }
+  __syncthreads();
+  const int fr = lane & 15, fk = lane >> 4;
+  const size_t tile = ((size_t)blockIdx.x * H + h) * N * dv;
+  if (MODE == 1) {
+    const float lal = la[n - 1];
+    if (tid < kSC) wgt[tid] = tid < n ? expf(lal - la[tid]) * dts[tid] : 0.0f;
+    __syncthreads();
+    for (int td = wave; td < NP / 16; td += 4) {
+      f32x4_t s[4];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) s[c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+      for (int k = 0; k < kSC; k += 4) {
+        const int j = k + fk;
+        const float a = Bs[j * NS + td * 16 + fr] * wgt[j];
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          s[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, Xs[j * kXS + c * 16 + fr], s[c], 0, 0, 0);
+      }
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int row = td * 16 + fk * 4 + r, col = col0 + c * 16 + fr;
+          if (row < N && col < dv) p.ws[tile + (size_t)row * dv + col] = s[c][r];
+        }
+    }
+    if (tid == 0 && blockIdx.z == 0) p.wdec[(size_t)blockIdx.x * H + h] = expf(lal);
+    return;
+  }
+  // ---- MODE 2: wave w owns tokens 16 w .. 16 w + 15
+  const int ti = wave;
+  {
+    f32x4_t acc[4];
+#pragma unroll
+    for (int tj = 0; tj < 4; ++tj) acc[tj] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    const float* qa = Cs + (ti * 16 + fr) * NS + fk;
+    const float* kb = Bs + fr * NS + fk;
+#pragma unroll 2
+    for (int k = 0; k < NP; k += 4) {
+      const float a = qa[k];
+#pragma unroll
+      for (int tj = 0; tj < 4; ++tj)
+        if (tj <= ti) acc[tj] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, kb[tj * 16 * NS + k], acc[tj], 0, 0, 0);
+    }
+#pragma unroll
+    for (int tj = 0; tj < 4; ++tj)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int i = ti * 16 + fk * 4 + r, j = tj * 16 + fr;
+        Gs[i * kGS + j] = j <= i ? acc[tj][r] * expf(la[i] - la[j]) * dts[j] : 0.0f;
+      }
+  }
+  f32x4_t o[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) o[c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const float* sp = p.ws + tile;  // the state at this chunk's start (after the carry)
+#pragma unroll 2
+  for (int k = 0; k < NP; k += 4) {
+    const float a = Cs[(ti * 16 + fr) * NS + k + fk];
+    const int krow = k + fk;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int col = col0 + c * 16 + fr;
+      const float sv = (krow < N && col < dv) ? sp[(size_t)krow * dv + col] : 0.0f;
+      o[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, sv, o[c], 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < 4; ++c)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) o[c][r] *= expf(la[ti * 16 + fk * 4 + r]);
+  __syncthreads();
+#pragma unroll 4
+  for (int k = 0; k < (ti + 1) * 16; k += 4) {
+    const float a = Gs[(ti * 16 + fr) * kGS + k + fk];
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+      o[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, Xs[(k + fk) * kXS + c * 16 + fr], o[c], 0, 0, 0);
+  }
+  const float Dh = p.D[h];
+#pragma unroll
+  for (int c = 0; c < 4; ++c)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int i = ti * 16 + fk * 4 + r, col = col0 + c * 16 + fr;
+      if (i < n && col < dv)
+        p.y[(size_t)(tc + i) * inner + (size_t)h * dv + col] = fmaf(Dh, Xs[i * kXS + c * 16 + fr], o[c][r]);
+    }
+}
+
+// grid (B, heads, ceil(N dv / 256)): one state element per thread walks its sequence's chunks: the workspace's local
+// sums become the states at the chunks' starts, and the state after the last chunk goes back to the slot
+__global__ void __launch_bounds__(256) ssd_carry_kernel(SsdArgs p) {
+  const int b = blockIdx.x, h = blockIdx.y;
+  const int e = blockIdx.z * 256 + threadIdx.x;
+  const int nd = p.N * p.dv;
+  if (e >= nd) return;
+  const int chunks = (p.seq_start[b + 1] - p.seq_start[b] + kSC - 1) / kSC;
+  float* st = p.state + ((size_t)p.seq_slot[b] * p.heads + h) * nd + e;
+  float s = p.seq_pos0[b] > 0 ? *st : 0.0f;
+  for (int c = 0; c < chunks; ++c) {
+    const size_t idx = ((size_t)b * p.max_chunks + c) * p.heads + h;
+    const float local = p.ws[idx * nd + e];
+    p.ws[idx * nd + e] = s;
+    s = fmaf(p.wdec[idx], s, local);
+  }
+  *st = s;
+}
+
+static size_t ssd_lds(int N) {
+  const int NP = (N + 15) / 16 * 16;
+  return sizeof(float) * ((size_t)2 * kSC * (NP + 2) + kSC * kXS + kSC * kGS + 3 * kSC);
+}
+
 // grid (T, groups): out[t][g n + i] = v / sqrt(mean_g(v^2) + eps) * w[g n + i], v = y * silu(z)
 __global__ void __launch_bounds__(256) gated_group_norm_kernel(const float* __restrict__ y, const float* __restrict__ z,
                                                                long ldz, const float* __restrict__ w, float eps,
@@ -199,13 +386,32 @@ extern "C" int lgs_conv_silu(const float* u, long ld, const void* w, const void*
 extern "C" int lgs_ssm_scan(const float* xbc, long ldx, const float* dt, long ldd, const float* dt_bias,
                             const float* A_log, const float* D, float* state, const int* seq_start,
                             const int* seq_slot, const int* seq_pos0, float* y, int B, int heads, int groups, int N,
-                            int dv, hipStream_t stream) {
+                            int dv, float* ws, float* wdec, int max_chunks, hipStream_t stream) {
   LGA_CHECK_ARG(xbc && dt && dt_bias && A_log && D && state && seq_start && seq_slot && seq_pos0 && y,
                 "lgs_ssm_scan: null pointer");
   LGA_CHECK_ARG(B > 0 && B <= 65535 && heads > 0 && heads <= 65535 && groups > 0 && heads % groups == 0,
                 "lgs_ssm_scan: heads must be a multiple of the groups");
   LGA_CHECK_ARG(N > 0 && N <= 256 && dv > 0, "lgs_ssm_scan: state size 1 to 256");
   LGA_CHECK_ARG(ldx >= (long)heads * dv + 2L * groups * N && ldd >= heads, "lgs_ssm_scan: rows shorter than their parts");
+  if (ws) {  // the prompt form
+    LGA_CHECK_ARG(wdec && max_chunks > 0 && N <= 128, "lgs_ssm_scan: the prompt form serves state sizes up to 128");
+    LGA_CHECK_ARG((long)B * max_chunks < (1L << 31) && (dv + 63) / 64 <= 65535, "lgs_ssm_scan: too many chunks");
+    lgs::SsdArgs p{xbc, ldx, dt, ldd, dt_bias, A_log, D, state, seq_start, seq_slot, seq_pos0, y, ws, wdec,
+                   heads, groups, N, dv, max_chunks};
+    const size_t lds = lgs::ssd_lds(N);
+    for (auto* fn : {lgs::ssd_chunk_kernel<1>, lgs::ssd_chunk_kernel<2>}) {
+      const hipError_t e = hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess) {
+        lga_set_error(hipGetErrorString(e));
+        return (int)e;
+      }
+    }
+    const dim3 grid(B * max_chunks, heads, (dv + 63) / 64);
+    lgs::ssd_chunk_kernel<1><<<grid, 256, lds, stream>>>(p);
+    lgs::ssd_carry_kernel<<<dim3(B, heads, (N * dv + 255) / 256), 256, 0, stream>>>(p);
+    lgs::ssd_chunk_kernel<2><<<grid, 256, lds, stream>>>(p);
+    LGA_LAUNCH_RETURN();
+  }
   lgs::ScanArgs p{xbc, ldx, dt, ldd, dt_bias, A_log, D, state, seq_start, seq_slot, seq_pos0, y, heads, groups, N, dv};
   const dim3 grid((dv + 63) / 64, heads, B);
   const int nr = (N + 3) / 4;

@@ -267,7 +267,8 @@ class SelectiveScan(InputReader):
         xbc = seq_ops.conv_silu(proj, base + inner, self.conv_w, self.conv_b, cache.conv, *tables,
                                 step.max_len or step.T)
         y = seq_ops.ssm_scan(xbc, proj, base + inner + self.channels, self.dt_bias, self.A_log, self.D, cache.s,
-                             *tables, heads=self.H, groups=self.G, N=self.N, dv=self.dv)
+                             *tables, heads=self.H, groups=self.G, N=self.N, dv=self.dv,
+                             max_len=step.max_len or step.T)
         g = seq_ops.gated_group_norm(y, proj, base, self.norm_w, groups=self.norm_groups, eps=self.eps,
                                      bf16_copy=_tiles16(step.T, self.w_o))
         W = x.shape[1]

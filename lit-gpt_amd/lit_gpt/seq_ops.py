@@ -53,7 +53,7 @@ SIGNATURES = {
     "lgs_diffattn": [_P, _L, _P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _F, _F, _F, _F,
                      _F, _P],
     "lgs_conv_silu": [_P, _L, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
-    "lgs_ssm_scan": [_P, _L, _P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
+    "lgs_ssm_scan": [_P, _L, _P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _I, _P],
     "lgs_gated_group_norm": [_P, _P, _L, _P, _F, _P, _P, _I, _I, _I, _P],
     "lgs_glu_clamped": [_P, _P, _L, _P, _I, _I, _I, _F, _F, _F, _P],
 }
@@ -473,9 +473,12 @@ def conv_silu(proj: torch.Tensor, off: int, weight: torch.Tensor, bias: torch.Te
 
 def ssm_scan(xbc: torch.Tensor, proj: torch.Tensor, dt_off: int, dt_bias: torch.Tensor, A_log: torch.Tensor,
              D: torch.Tensor, state: torch.Tensor, seq_start: torch.Tensor, seq_slot: torch.Tensor,
-             seq_pos0: torch.Tensor, *, heads: int, groups: int, N: int, dv: int) -> torch.Tensor:
+             seq_pos0: torch.Tensor, *, heads: int, groups: int, N: int, dv: int, max_len: int = 0,
+             chunked: Optional[bool] = None) -> torch.Tensor:
     """The selective scan over a packed batch: xbc (T, heads dv + 2 groups N) after the convolution, raw step sizes
-    in the ``heads`` columns of ``proj`` at ``dt_off``; state (slots, heads, N, dv) fp32. Returns y (T, heads dv)."""
+    in the ``heads`` columns of ``proj`` at ``dt_off``; state (slots, heads, N, dv) fp32. Returns y (T, heads dv).
+    ``chunked`` picks the prompt form (64-token chunks as matrix products, all chunks side by side; N <= 128) over
+    the token-by-token walk; by default steps in which a sequence brings more than 16 tokens (``max_len``) take it."""
     T, ldx = xbc.shape
     B = seq_slot.numel()
     if ldx != heads * dv + 2 * groups * N or tuple(state.shape[1:]) != (heads, N, dv) or proj.shape[0] != T:
@@ -483,11 +486,21 @@ def ssm_scan(xbc: torch.Tensor, proj: torch.Tensor, dt_off: int, dt_bias: torch.
     if dt_off + heads > proj.shape[1] or min(dt_bias.numel(), A_log.numel(), D.numel()) != heads:
         raise ValueError("ssm_scan: per-head parameters")
     y = torch.empty(T, heads * dv, dtype=F32, device=xbc.device)
+    if chunked is None:
+        chunked = max_len > 16 and N <= 128
+    ws, wdec, max_chunks = None, None, 0
+    if chunked:
+        if not 0 < max_len <= T or N > 128:
+            raise ValueError("ssm_scan: the prompt form needs the longest sequence's token count and N <= 128")
+        max_chunks = (max_len + 63) // 64
+        ws = torch.empty(B * max_chunks * heads * N * dv, dtype=F32, device=xbc.device)
+        wdec = torch.empty(B * max_chunks * heads, dtype=F32, device=xbc.device)
     _check(load_library().lgs_ssm_scan(_dev(xbc, "xbc", F32), ldx, _dev(proj, "proj", F32) + 4 * dt_off,
                                        proj.shape[1], _dev(dt_bias, "dt_bias", F32), _dev(A_log, "A_log", F32),
                                        _dev(D, "D", F32), _dev(state, "state", F32), _dev(seq_start, "seq_start", I32),
                                        _dev(seq_slot, "seq_slot", I32), _dev(seq_pos0, "seq_pos0", I32), y.data_ptr(),
-                                       B, heads, groups, N, dv, _stream()))
+                                       B, heads, groups, N, dv, _opt(ws, "ws", F32), _opt(wdec, "wdec", F32),
+                                       max_chunks, _stream()))
     return y
 
 

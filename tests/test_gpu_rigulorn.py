@@ -376,6 +376,61 @@ def test_state_carries_a_far_token():
         assert rel_err(engine_logits(model, [toks], [cuts])[0], whole).max() < SAME
 
 
+def plain_scan(xbc, dt_raw, dt_bias, A_log, D, heads, groups, N, dv, S0):
+    """Token by token in float64; returns y (T, heads dv) and the final state (heads, N, dv)."""
+    T = xbc.shape[0]
+    inner = heads * dv
+    x = xbc[:, :inner].double().view(T, heads, dv)
+    Bm = xbc[:, inner:inner + groups * N].double().view(T, groups, N)
+    Cm = xbc[:, inner + groups * N:].double().view(T, groups, N)
+    dt = orc.softplus(dt_raw.double() + dt_bias.double())
+    a = torch.exp(-torch.exp(A_log.double()) * dt)
+    S = S0.double().clone()
+    y = torch.zeros(T, heads, dv, dtype=torch.float64)
+    for t in range(T):
+        for h in range(heads):
+            g = h // (heads // groups)
+            S[h] = a[t, h] * S[h] + dt[t, h] * torch.outer(Bm[t, g], x[t, h])
+            y[t, h] = S[h].T @ Cm[t, g] + D[h].double() * x[t, h]
+    return y.reshape(T, inner), S
+
+
+@pytest.mark.parametrize("heads,groups,N,dv", [(4, 2, 16, 8), (2, 1, 40, 70), (3, 3, 128, 64), (2, 2, 5, 3)])
+def test_scan_prompt_form_against_token_walk(heads, groups, N, dv):
+    """Several sequences of unequal lengths (one chunk, several chunks, a chunk's edge) in one step, continued from a
+    state in the slot or started anew over a slot with stale contents; both forms against float64."""
+    from lit_gpt import seq_ops
+    from lit_gpt.mixers import StepBatch
+
+    dev = torch.device("cuda", 0)
+    g = torch.Generator().manual_seed(N + dv)
+    lens, pos0 = [64, 150, 17, 65, 1], [0, 9, 3, 0, 7]
+    T, inner = sum(lens), heads * dv
+    xbc = torch.randn(T, inner + 2 * groups * N, generator=g) * 0.5
+    raw = torch.randn(T, heads + 2, generator=g)
+    dt_bias, A_log, D = torch.randn(heads, generator=g) - 1.0, torch.randn(heads, generator=g), torch.randn(heads, generator=g)
+    stale = torch.randn(len(lens) + 1, heads, N, dv, generator=g)
+    want_y, want_s, at = [], [], 0
+    for i, (n, p0) in enumerate(zip(lens, pos0)):
+        S0 = stale[i] if p0 > 0 else torch.zeros(heads, N, dv)
+        y, S = plain_scan(xbc[at:at + n], raw[at:at + n, 2:], dt_bias, A_log, D, heads, groups, N, dv, S0)
+        want_y.append(y)
+        want_s.append(S)
+        at += n
+    want_y = torch.cat(want_y)
+    step = StepBatch.build([(i, p0, [0] * n) for i, (n, p0) in enumerate(zip(lens, pos0))], dev)
+    for chunked in (False, True):
+        state = stale.to(dev).clone()
+        y = seq_ops.ssm_scan(xbc.to(dev), raw.to(dev), 2, dt_bias.to(dev), A_log.to(dev), D.to(dev), state,
+                             step.seq_start, step.seq_slot, step.seq_pos0, heads=heads, groups=groups, N=N, dv=dv,
+                             max_len=max(lens), chunked=chunked)
+        scale = want_y.abs().max()
+        assert (y.double().cpu() - want_y).abs().max() < 2e-5 * scale, chunked
+        for i, S in enumerate(want_s):
+            assert (state[i].double().cpu() - S).abs().max() < 2e-5 * S.abs().max().clamp_min(1.0), (chunked, i)
+        assert torch.equal(state[-1].cpu(), stale[-1])
+
+
 # ------------------------------------------------------------------------------------------------ small operations
 @pytest.mark.parametrize("s", [1, 2, 3, 8])
 def test_streams_step(s):
