@@ -202,6 +202,20 @@ __global__ void __launch_bounds__(256) ssd_chunk_kernel(SsdArgs p) {
   float* la = Gs + kSC * kGS;
   float* dts = la + kSC;
   float* wgt = dts + kSC;
+  const int fr = lane & 15, fk = lane >> 4;
+  const size_t tile = ((size_t)blockIdx.x * H + h) * N * dv;
+  // MODE 2: this lane's share of the state at the chunk's start (the B operand of C S0), fetched before anything
+  // else so that its latency passes under the staging and the score product (one wave per SIMD: nothing else hides it)
+  float sv[32][4];
+  if (MODE == 2) {
+#pragma unroll
+    for (int kk = 0; kk < 32; ++kk)
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int krow = kk * 4 + fk, col = col0 + c * 16 + fr;
+        sv[kk][c] = (krow < N && col < dv) ? p.ws[tile + (size_t)krow * dv + col] : 0.0f;
+      }
+  }
   if (wave == 0) {
     float d = 0.0f, l = 0.0f;
     if (lane < n) {
@@ -228,8 +242,6 @@ __global__ void __launch_bounds__(256) ssd_chunk_kernel(SsdArgs p) {
     Xs[row * kXS + c] = (row < n && col0 + c < dv) ? p.xbc[(size_t)(tc + row) * p.ldx + (size_t)h * dv + col0 + c] : 0.0f;
   }
   __syncthreads();
-  const int fr = lane & 15, fk = lane >> 4;
-  const size_t tile = ((size_t)blockIdx.x * H + h) * N * dv;
   if (MODE == 1) {
     const float lal = la[n - 1];
     if (tid < kSC) wgt[tid] = tid < n ? expf(lal - la[tid]) * dts[tid] : 0.0f;
@@ -283,16 +295,12 @@ __global__ void __launch_bounds__(256) ssd_chunk_kernel(SsdArgs p) {
   f32x4_t o[4];
 #pragma unroll
   for (int c = 0; c < 4; ++c) o[c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  const float* sp = p.ws + tile;  // the state at this chunk's start (after the carry)
-#pragma unroll 2
-  for (int k = 0; k < NP; k += 4) {
-    const float a = Cs[(ti * 16 + fr) * NS + k + fk];
-    const int krow = k + fk;
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const int col = col0 + c * 16 + fr;
-      const float sv = (krow < N && col < dv) ? sp[(size_t)krow * dv + col] : 0.0f;
-      o[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, sv, o[c], 0, 0, 0);
+  for (int kk = 0; kk < 32; ++kk) {
+    if (kk * 4 < NP) {
+      const float a = Cs[(ti * 16 + fr) * NS + kk * 4 + fk];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) o[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, sv[kk][c], o[c], 0, 0, 0);
     }
   }
 #pragma unroll

@@ -92,6 +92,84 @@ __global__ void __launch_bounds__(256) streams_step_kernel(StreamArgs p) {
   }
 }
 
+// The same step with a token's columns in registers: thread i owns columns i + 256 c, c < CPT (W <= 256 CPT), of
+// SMAX >= s streams. All loads are issued before the first use and the normed read is written from registers, so a
+// one-token step is one round trip to memory instead of one per column block.
+template <int SMAX, int CPT>
+__global__ void __launch_bounds__(256) streams_step_reg_kernel(StreamArgs p) {
+  __shared__ float red[4];
+  __shared__ float cm[kMaxStreams * kMaxStreams], cb[kMaxStreams], ca[kMaxStreams];
+  const int s = p.s, W = p.W;
+  if (threadIdx.x < s * s) cm[threadIdx.x] = p.mix ? p.mix[threadIdx.x] : 0.0f;
+  if (threadIdx.x < s) {
+    cb[threadIdx.x] = p.out ? p.out[threadIdx.x] : 0.0f;
+    ca[threadIdx.x] = p.in ? p.in[threadIdx.x] : 0.0f;
+  }
+  float* xt = p.x + (size_t)blockIdx.x * s * W;
+  const float* yt = p.y ? p.y + (size_t)blockIdx.x * W : nullptr;
+  float v[SMAX][CPT], y[CPT], nw[CPT];
+#pragma unroll
+  for (int c = 0; c < CPT; ++c) {
+    const int i = threadIdx.x + 256 * c;
+#pragma unroll
+    for (int j = 0; j < SMAX; ++j) v[j][c] = (j < s && i < W) ? xt[(size_t)j * W + i] : 0.0f;
+    y[c] = (yt && i < W) ? yt[i] : 0.0f;
+    nw[c] = (p.in && p.w && i < W) ? p.w[i] : 1.0f;
+  }
+  __syncthreads();
+  float u[CPT], ss = 0.0f;
+#pragma unroll
+  for (int c = 0; c < CPT; ++c) {
+    const int i = threadIdx.x + 256 * c;
+    if (yt) {
+      float nv[SMAX];
+#pragma unroll
+      for (int j = 0; j < SMAX; ++j) {
+        float acc = 0.0f;
+#pragma unroll
+        for (int k = 0; k < SMAX; ++k)
+          if (k < s && j < s) acc = fmaf(cm[k * s + j], v[k][c], acc);
+        nv[j] = j < s ? fmaf(cb[j], y[c], acc) : 0.0f;
+      }
+#pragma unroll
+      for (int j = 0; j < SMAX; ++j) {
+        v[j][c] = nv[j];
+        if (j < s && i < W) xt[(size_t)j * W + i] = nv[j];
+      }
+    }
+    float a = 0.0f;
+#pragma unroll
+    for (int j = 0; j < SMAX; ++j)
+      if (j < s) a = fmaf(ca[j], v[j][c], a);
+    u[c] = a;
+    ss = fmaf(a, a, ss);
+  }
+  if (!p.in) return;
+  float rstd = 1.0f;
+  if (p.w) {
+    ss = block_sum_256(ss, red);
+    rstd = 1.0f / sqrtf(ss / (float)W + p.eps);
+  }
+#pragma unroll
+  for (int c = 0; c < CPT; ++c) {
+    const int i = threadIdx.x + 256 * c;
+    if (i >= W) continue;
+    const size_t at = (size_t)blockIdx.x * W + i;
+    const float r = p.w ? u[c] * rstd * nw[c] : u[c];
+    p.h[at] = r;
+    if (p.h16) p.h16[at] = f2bf(r);
+  }
+}
+
+template <int SMAX>
+static bool streams_step_reg(const StreamArgs& p, int T, hipStream_t stream) {
+  if (p.W <= 1024) streams_step_reg_kernel<SMAX, 4><<<T, 256, 0, stream>>>(p);
+  else if (p.W <= 2048) streams_step_reg_kernel<SMAX, 8><<<T, 256, 0, stream>>>(p);
+  else if (p.W <= 4096 && SMAX <= 4) streams_step_reg_kernel<SMAX, 16><<<T, 256, 0, stream>>>(p);
+  else return false;
+  return true;
+}
+
 }  // namespace lgs
 
 extern "C" int lgs_embed_streams(const int* tokens, const void* table, int w_f32, float scale, float* x, int T, int W,
@@ -113,6 +191,11 @@ extern "C" int lgs_streams_step(float* x, const float* y, const float* mix, cons
   LGA_CHECK_ARG(norm_w || !h_bf16, "lgs_streams_step: the bf16 copy is made by the norm");
   LGA_CHECK_ARG(y || in, "lgs_streams_step: nothing to do");
   lgs::StreamArgs p{x, y, mix, out, in, norm_w, h, (uint16_t*)h_bf16, eps, W, streams};
-  lgs::streams_step_kernel<<<T, 256, 0, stream>>>(p);
+  bool done;
+  if (streams == 1) done = lgs::streams_step_reg<1>(p, T, stream);
+  else if (streams == 2) done = lgs::streams_step_reg<2>(p, T, stream);
+  else if (streams <= 4) done = lgs::streams_step_reg<4>(p, T, stream);
+  else done = lgs::streams_step_reg<8>(p, T, stream);
+  if (!done) lgs::streams_step_kernel<<<T, 256, 0, stream>>>(p);  // wide rows: column blocks one after the other
   LGA_LAUNCH_RETURN();
 }
