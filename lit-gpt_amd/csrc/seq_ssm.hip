@@ -164,7 +164,7 @@ __global__ void __launch_bounds__(256) ssm_scan_kernel(ScanArgs p) {
 // MODE 1, grid (B * max_chunks, heads, ceil(dv / 64)): the second term of S' of every chunk -> workspace, the chunk's
 // whole decay -> wdec. ssd_carry_kernel turns these into the state at each chunk's start (an elementwise recurrence
 // over the chunks, which also leaves the final state in the slot). MODE 2: the outputs of every chunk.
-// LDS (floats): C, B [64][NP + 2], x [64][80], scores [64][66], l, dt, weights [64] each; N <= 128.
+// LDS (floats): C, B [64][NP + 4], x [64][80], scores [64][66], l, dt, weights [64] each; N <= 128.
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 constexpr int kSC = 64, kXS = 80, kGS = 66;
 
@@ -194,7 +194,7 @@ __global__ void __launch_bounds__(256) ssd_chunk_kernel(SsdArgs p) {
   const int n = min(kSC, t1 - tc);
   const int N = p.N, dv = p.dv, H = p.heads, inner = H * dv;
   const int g = h / (H / p.groups);
-  const int NP = (N + 15) / 16 * 16, NS = NP + 2;
+  const int NP = (N + 15) / 16 * 16, NS = NP + 4;
   float* Cs = lds;
   float* Bs = Cs + kSC * NS;
   float* Xs = Bs + kSC * NS;
@@ -230,16 +230,34 @@ __global__ void __launch_bounds__(256) ssd_chunk_kernel(SsdArgs p) {
     la[lane] = l;
     dts[lane] = d;
   }
-  for (int i = tid; i < kSC * NP; i += 256) {
-    const int row = i / NP, k = i - row * NP;
-    const bool in = row < n && k < N;
-    const size_t at = (size_t)(tc + row) * p.ldx + inner + (size_t)g * N + k;
-    Bs[row * NS + k] = in ? p.xbc[at] : 0.0f;
-    if (MODE == 2) Cs[row * NS + k] = in ? p.xbc[at + (size_t)p.groups * N] : 0.0f;
-  }
-  for (int i = tid; i < kSC * 64; i += 256) {
-    const int row = i >> 6, c = i & 63;
-    Xs[row * kXS + c] = (row < n && col0 + c < dv) ? p.xbc[(size_t)(tc + row) * p.ldx + (size_t)h * dv + col0 + c] : 0.0f;
+  const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (((N | dv | inner) & 3) == 0 && (p.ldx & 3) == 0) {  // 16-byte loads and LDS stores (NS is a multiple of 4)
+    const int q = NP / 4;
+    for (int i = tid; i < kSC * q; i += 256) {
+      const int row = i / q, k = (i - row * q) * 4;
+      const bool in = row < n && k < N;
+      const float* at = p.xbc + (size_t)(tc + row) * p.ldx + inner + (size_t)g * N + k;
+      *(float4*)(Bs + row * NS + k) = in ? *(const float4*)at : zero4;
+      if (MODE == 2) *(float4*)(Cs + row * NS + k) = in ? *(const float4*)(at + (size_t)p.groups * N) : zero4;
+    }
+    for (int i = tid; i < kSC * 16; i += 256) {
+      const int row = i >> 4, c = (i & 15) * 4;
+      const bool in = row < n && col0 + c < dv;
+      *(float4*)(Xs + row * kXS + c) =
+          in ? *(const float4*)(p.xbc + (size_t)(tc + row) * p.ldx + (size_t)h * dv + col0 + c) : zero4;
+    }
+  } else {
+    for (int i = tid; i < kSC * NP; i += 256) {
+      const int row = i / NP, k = i - row * NP;
+      const bool in = row < n && k < N;
+      const size_t at = (size_t)(tc + row) * p.ldx + inner + (size_t)g * N + k;
+      Bs[row * NS + k] = in ? p.xbc[at] : 0.0f;
+      if (MODE == 2) Cs[row * NS + k] = in ? p.xbc[at + (size_t)p.groups * N] : 0.0f;
+    }
+    for (int i = tid; i < kSC * 64; i += 256) {
+      const int row = i >> 6, c = i & 63;
+      Xs[row * kXS + c] = (row < n && col0 + c < dv) ? p.xbc[(size_t)(tc + row) * p.ldx + (size_t)h * dv + col0 + c] : 0.0f;
+    }
   }
   __syncthreads();
   if (MODE == 1) {
@@ -347,7 +365,7 @@ __global__ void __launch_bounds__(256) ssd_carry_kernel(SsdArgs p) {
 
 static size_t ssd_lds(int N) {
   const int NP = (N + 15) / 16 * 16;
-  return sizeof(float) * ((size_t)2 * kSC * (NP + 2) + kSC * kXS + kSC * kGS + 3 * kSC);
+  return sizeof(float) * ((size_t)2 * kSC * (NP + 4) + kSC * kXS + kSC * kGS + 3 * kSC);
 }
 
 // grid (T, groups): out[t][g n + i] = v / sqrt(mean_g(v^2) + eps) * w[g n + i], v = y * silu(z)
