@@ -90,6 +90,10 @@ struct AttnArgs {
 };
 
 constexpr int kKeyTile = 256;
+// row stride of the score / weight tile in LDS, [key][(query, map)]: a key's weights for all queries and maps lie
+// side by side, so the value phase fetches them with 16-byte reads
+template <int QT>
+constexpr int score_stride() { return QT == 1 ? 4 : 2 * QT + 4; }
 
 // o = a1 / l1 - lambda a2 / l2 over the head, unit RMS, times post. Called by all 256 threads; thread c < dv owns
 // column c (dv <= 256).
@@ -106,7 +110,7 @@ __device__ __forceinline__ void diff_finish(float a1, float a2, float l1, float 
   }
 }
 
-// grid (B * tiles, H, splits). LDS: queries [QT][2 d], scores / weights [2 QT][256], per (query, map) the running
+// grid (B * tiles, H, splits). LDS: queries [QT][2 d], scores / weights [256][2 QT + 4], per (query, map) the running
 // maximum, normaliser and the rescale of the current tile, and the cross-subset sums of the value phase.
 template <int QT, bool CF32>
 __global__ void __launch_bounds__(256) diffattn_kernel(AttnArgs p) {
@@ -114,8 +118,9 @@ __global__ void __launch_bounds__(256) diffattn_kernel(AttnArgs p) {
   __shared__ float red[4];
   const int d = p.d, dv = p.dv, d2 = 2 * d;
   float* qs = lds;                       // [QT][d2]
-  float* sc = qs + QT * d2;              // [2 QT][kKeyTile]
-  float* mrow = sc + 2 * QT * kKeyTile;  // [2 QT] running maximum
+  constexpr int SCS = score_stride<QT>();
+  float* sc = qs + QT * d2;              // [kKeyTile][SCS]: scores, then weights, of key x (query, map)
+  float* mrow = sc + kKeyTile * SCS;     // [2 QT] running maximum
   float* lrow = mrow + 2 * QT;           // [2 QT] running normaliser
   float* arow = lrow + 2 * QT;           // [2 QT] rescale of what was summed before this tile
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -196,18 +201,18 @@ __global__ void __launch_bounds__(256) diffattn_kernel(AttnArgs p) {
         for (int m = 0; m < 2; ++m) {
           float v = s[i][m] * p.scale;
           if (p.cap > 0.0f) v = p.cap * tanhf(v / p.cap);
-          sc[(2 * i + m) * kKeyTile + tid] = see ? v : -INFINITY;
+          sc[tid * SCS + 2 * i + m] = see ? v : -INFINITY;
         }
       }
     }
     __syncthreads();
     // ---- online softmax: wave w owns rows w, w + 4, ... of the 2 QT (query, map) rows
     for (int r = wave; r < 2 * QT; r += 4) {
-      float* srow = sc + r * kKeyTile;
+      float* srow = sc + r;
       float v[4], mx = -INFINITY;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        v[e] = srow[lane + 64 * e];
+        v[e] = srow[(lane + 64 * e) * SCS];
         mx = fmaxf(mx, v[e]);
       }
       mx = wave_max(mx);
@@ -216,7 +221,7 @@ __global__ void __launch_bounds__(256) diffattn_kernel(AttnArgs p) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const float w = mn == -INFINITY ? 0.0f : expf(v[e] - mn);  // (a masked key: exp(-inf) = 0)
-        srow[lane + 64 * e] = w;
+        srow[(lane + 64 * e) * SCS] = w;
         sum += w;
       }
       sum = wave_sum(sum);
@@ -236,12 +241,24 @@ __global__ void __launch_bounds__(256) diffattn_kernel(AttnArgs p) {
         acc[i][1] *= arow[2 * i + 1];
       }
       if (col < dv) {
+#pragma unroll 4
         for (int j = ks; j < nk; j += KS) {
           const float v = cload<CF32>(p.cache_v, ((slot * p.S + k0 + j) * p.G + g) * dv + col);
+          float w[2 * QT];
+          if (QT == 1) {
+            const float2 t = *(const float2*)(sc + j * SCS);
+            w[0] = t.x, w[1] = t.y;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 2 * QT; e += 4) {
+              const float4 t = *(const float4*)(sc + j * SCS + e);
+              w[e] = t.x, w[e + 1] = t.y, w[e + 2] = t.z, w[e + 3] = t.w;
+            }
+          }
 #pragma unroll
           for (int i = 0; i < QT; ++i) {
-            acc[i][0] = fmaf(sc[(2 * i) * kKeyTile + j], v, acc[i][0]);
-            acc[i][1] = fmaf(sc[(2 * i + 1) * kKeyTile + j], v, acc[i][1]);
+            acc[i][0] = fmaf(w[2 * i], v, acc[i][0]);
+            acc[i][1] = fmaf(w[2 * i + 1], v, acc[i][1]);
           }
         }
       }
@@ -249,7 +266,7 @@ __global__ void __launch_bounds__(256) diffattn_kernel(AttnArgs p) {
     __syncthreads();
   }
   // ---- sum the key subsets (fixed order), then finish or leave the split's partial result
-  float* xs = sc;  // [KS][2 QT][ncol] <= 256 * 2 QT floats
+  float* xs = sc;  // [KS][2 QT][ncol] = 256 * 2 QT floats <= the score tile
   if (KS > 1) {
 #pragma unroll
     for (int i = 0; i < QT; ++i) {
@@ -307,7 +324,9 @@ __global__ void __launch_bounds__(256) diffattn_combine_kernel(AttnArgs p, int s
 }
 
 template <int QT>
-static size_t diffattn_lds(int d) { return sizeof(float) * ((size_t)QT * 2 * d + 2 * QT * kKeyTile + 6 * QT); }
+static size_t diffattn_lds(int d) {
+  return sizeof(float) * ((size_t)QT * 2 * d + (size_t)kKeyTile * score_stride<QT>() + 6 * QT);
+}
 
 template <int QT>
 static int diffattn_launch(const AttnArgs& p, int cache_f32, dim3 grid, hipStream_t stream) {

@@ -95,9 +95,11 @@ __global__ void __launch_bounds__(256) streams_step_kernel(StreamArgs p) {
 // The same step with a token's columns in registers: thread i owns columns i + 256 c, c < CPT (W <= 256 CPT), of
 // SMAX >= s streams. All loads are issued before the first use and the normed read is written from registers, so a
 // one-token step is one round trip to memory instead of one per column block.
-template <int SMAX, int CPT>
-__global__ void __launch_bounds__(256) streams_step_reg_kernel(StreamArgs p) {
-  __shared__ float red[4];
+// (NT threads per token: 256 for prompts, 1024 for steps of a few tokens, whose one workgroup per token is then
+// four times shorter.)
+template <int SMAX, int CPT, int NT>
+__global__ void __launch_bounds__(NT) streams_step_reg_kernel(StreamArgs p) {
+  __shared__ float red[NT / 64];
   __shared__ float cm[kMaxStreams * kMaxStreams], cb[kMaxStreams], ca[kMaxStreams];
   const int s = p.s, W = p.W;
   if (threadIdx.x < s * s) cm[threadIdx.x] = p.mix ? p.mix[threadIdx.x] : 0.0f;
@@ -110,7 +112,7 @@ __global__ void __launch_bounds__(256) streams_step_reg_kernel(StreamArgs p) {
   float v[SMAX][CPT], y[CPT], nw[CPT];
 #pragma unroll
   for (int c = 0; c < CPT; ++c) {
-    const int i = threadIdx.x + 256 * c;
+    const int i = threadIdx.x + NT * c;
 #pragma unroll
     for (int j = 0; j < SMAX; ++j) v[j][c] = (j < s && i < W) ? xt[(size_t)j * W + i] : 0.0f;
     y[c] = (yt && i < W) ? yt[i] : 0.0f;
@@ -120,7 +122,7 @@ __global__ void __launch_bounds__(256) streams_step_reg_kernel(StreamArgs p) {
   float u[CPT], ss = 0.0f;
 #pragma unroll
   for (int c = 0; c < CPT; ++c) {
-    const int i = threadIdx.x + 256 * c;
+    const int i = threadIdx.x + NT * c;
     if (yt) {
       float nv[SMAX];
 #pragma unroll
@@ -147,12 +149,17 @@ __global__ void __launch_bounds__(256) streams_step_reg_kernel(StreamArgs p) {
   if (!p.in) return;
   float rstd = 1.0f;
   if (p.w) {
-    ss = block_sum_256(ss, red);
+    ss = wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    ss = 0.0f;
+#pragma unroll
+    for (int w = 0; w < NT / 64; ++w) ss += red[w];
     rstd = 1.0f / sqrtf(ss / (float)W + p.eps);
   }
 #pragma unroll
   for (int c = 0; c < CPT; ++c) {
-    const int i = threadIdx.x + 256 * c;
+    const int i = threadIdx.x + NT * c;
     if (i >= W) continue;
     const size_t at = (size_t)blockIdx.x * W + i;
     const float r = p.w ? u[c] * rstd * nw[c] : u[c];
@@ -163,9 +170,16 @@ __global__ void __launch_bounds__(256) streams_step_reg_kernel(StreamArgs p) {
 
 template <int SMAX>
 static bool streams_step_reg(const StreamArgs& p, int T, hipStream_t stream) {
-  if (p.W <= 1024) streams_step_reg_kernel<SMAX, 4><<<T, 256, 0, stream>>>(p);
-  else if (p.W <= 2048) streams_step_reg_kernel<SMAX, 8><<<T, 256, 0, stream>>>(p);
-  else if (p.W <= 4096 && SMAX <= 4) streams_step_reg_kernel<SMAX, 16><<<T, 256, 0, stream>>>(p);
+  if (T <= 32 && p.W > 512) {
+    if (p.W <= 2048) streams_step_reg_kernel<SMAX, 2, 1024><<<T, 1024, 0, stream>>>(p);
+    else if (p.W <= 4096) streams_step_reg_kernel<SMAX, 4, 1024><<<T, 1024, 0, stream>>>(p);
+    else if (p.W <= 8192) streams_step_reg_kernel<SMAX, 8, 1024><<<T, 1024, 0, stream>>>(p);
+    else return false;
+    return true;
+  }
+  if (p.W <= 1024) streams_step_reg_kernel<SMAX, 4, 256><<<T, 256, 0, stream>>>(p);
+  else if (p.W <= 2048) streams_step_reg_kernel<SMAX, 8, 256><<<T, 256, 0, stream>>>(p);
+  else if (p.W <= 4096 && SMAX <= 4) streams_step_reg_kernel<SMAX, 16, 256><<<T, 256, 0, stream>>>(p);
   else return false;
   return true;
 }

@@ -432,14 +432,15 @@ def test_scan_prompt_form_against_token_walk(heads, groups, N, dv):
 
 
 # ------------------------------------------------------------------------------------------------ small operations
-@pytest.mark.parametrize("s,W", [(1, 300), (2, 300), (3, 1100), (8, 300), (4, 3000), (8, 3000), (3, 5000)])
-def test_streams_step(s, W):
-    """Narrow rows live in registers (by stream count and width), wide ones go column block by column block."""
+@pytest.mark.parametrize("T", [5, 40])
+@pytest.mark.parametrize("s,W", [(1, 300), (2, 300), (3, 1100), (8, 300), (4, 3000), (8, 3000), (3, 5000), (2, 9000)])
+def test_streams_step(s, W, T):
+    """Narrow rows live in registers (by stream count, width and row count), wide ones go column block by column
+    block."""
     from lit_gpt import seq_ops
 
     dev = torch.device("cuda", 0)
     g = torch.Generator().manual_seed(s)
-    T = 5
     x = torch.randn(T, s, W, generator=g)
     y, mix, out, read = torch.randn(T, W, generator=g), torch.randn(s, s, generator=g), torch.randn(s, generator=g), \
         torch.randn(s, generator=g)
