@@ -310,7 +310,7 @@ class LayeredConfig:
                               diff=float(m.get("diff", 0.0)), softcap=float(m.get("softcap") or 0.0),
                               mask_size=int(mask.get("size") or 0),
                               kv_from=int(m["kv_from"]) if m.get("kv_from") is not None else None,
-                              conv=int(m.get("conv", 0)), groups=int(m.get("groups", 0)),
+                              conv=int(m.get("conv", 0)), groups=int(m.get("groups", 1)),
                               norm_groups=int(m.get("norm_groups", 1)), state=int(m.get("state", 0)))
             f = entry.get("mlp")
             if f is None:

@@ -5,7 +5,7 @@ launch on torch's current HIP stream (capturable into a HIP graph) and raise on 
 no CPU path. Activations are fp32; a weight is a bf16 or an fp32 tensor and its dtype picks the kernel: bf16 weights
 take the activation rounded to bf16 with fp32 sums (MFMA tiles, streaming GEMVs), fp32 weights run plain fp32 FMA.
 
-The library is separate from ``liblitgpt_amd.so`` so that serving a layered model compiles four small sources only;
+The library is separate from ``liblitgpt_amd.so`` so that serving a layered model compiles a few small sources only;
 ``build_library`` runs that ``make`` target when the library is missing.
 """
 
