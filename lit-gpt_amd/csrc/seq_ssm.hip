@@ -7,7 +7,7 @@
 //                        S <- a S + dt B x^T (S is N x dv, fp32, one per cache slot), y = S^T C + D x;
 //                        heads share B and C in groups. Token by token (decode, short portions), or for prompts
 //                        in chunks of 64 tokens as fp32 matrix products with the chunks side by side
-//   lgs_gated_group_norm out = unit_rms_per_group(y * silu(z)) * w: the gate comes before the norm
+//   lgs_gated_group_norm out = unit_rms_per_group(y * silu(z)) * w: gating first, the grouped norm on the gated values
 #include "seq_common.h"
 
 namespace lgs {

@@ -177,7 +177,7 @@ class LatentAttention(InputReader):
 
 class DiffAttention(InputReader):
     """Differential softmax attention with grouped key / value heads. Every query head carries two maps (the q and k
-    rows of a head are laid out [map 1 | map 2], ``dim`` each); both attend over the same values and are combined as
+    rows of a head hold map 1 then map 2, ``dim`` rows each); both attend over the same values and are combined as
     o = a1 - lambda a2 with lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + diff (one number per layer), after which the
     head's output is divided by its root mean square and scaled by 1 - diff. Scores (q . k) * scale pass an optional
     tanh soft cap; rotary positions on interleaved pairs (2i, 2i + 1) of the first rot.dims dims of every map; a
@@ -229,7 +229,7 @@ class DiffAttention(InputReader):
 
 
 class SelectiveScan(InputReader):
-    """Selective state-space mixer in the Mamba-2 form. One input projection laid out [z | x | B | C | dt] (inner =
+    """Selective state-space mixer in the Mamba-2 form. One input projection whose rows are ordered [z | x | B | C | dt] (inner =
     heads * vdim gate and value columns, groups * state columns each for B and C, one step size per head); x, B and C
     pass a short causal per-channel convolution and silu; dt = softplus(dt + bias); per head (heads share B and C in
     groups) S_t = exp(-exp(A_log) dt_t) S_{t-1} + dt_t B_t x_t^T, y_t = S_t^T C_t + D x_t; y is gated with silu(z),

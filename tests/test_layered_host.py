@@ -254,7 +254,7 @@ def test_rigulorn_plain_implementation_is_causal_and_chunked():
     b = orc.forward(only, w1, other)
     assert torch.allclose(a[5:], b[5:], atol=1e-12) and not torch.allclose(a[4], b[4], atol=1e-6)
     assert orc.visible(9, 5, {"size": 5}) and not orc.visible(9, 4, {"size": 5}) and not orc.visible(4, 5, None)
-    # the convolution's last column is the current token's
+    # a kernel that is 1 in column taps - 1 and 0 elsewhere copies its input
     u = torch.arange(6.0, dtype=torch.float64).view(6, 1)
     got = orc.causal_conv(u, torch.tensor([[0.0, 0.0, 1.0]], dtype=torch.float64), torch.zeros(1, dtype=torch.float64))
     assert torch.equal(got, u)
