@@ -349,7 +349,8 @@ extern "C" int lgs_diffattn_prepare(float* proj, long ld, int q_off, int k_off, 
                                     int cache_f32, const float* inv_freq, const int* slot, const int* pos, int T, int H,
                                     int G, int d, int dv, int rot_dims, int max_seq, hipStream_t stream) {
   LGA_CHECK_ARG(proj && slot && pos && T > 0, "lgs_diffattn_prepare: bad arguments");
-  LGA_CHECK_ARG(H > 0 && G > 0 && H % G == 0 && d > 0 && dv > 0, "lgs_diffattn_prepare: heads must be a multiple of the key heads");
+  LGA_CHECK_ARG(H > 0 && G > 0 && H % G == 0 && d > 0 && dv > 0,
+                "lgs_diffattn_prepare: heads must be a multiple of the key heads");
   LGA_CHECK_ARG(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= d && (rot_dims == 0 || inv_freq),
                 "lgs_diffattn_prepare: rotary dims");
   LGA_CHECK_ARG(k_off < 0 || (cache_k && cache_v && v_off >= 0 && max_seq > 0), "lgs_diffattn_prepare: cache");

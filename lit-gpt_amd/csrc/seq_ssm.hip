@@ -451,7 +451,8 @@ extern "C" int lgs_ssm_scan(const float* xbc, long ldx, const float* dt, long ld
 extern "C" int lgs_gated_group_norm(const float* y, const float* z, long ldz, const float* w, float eps, float* out,
                                     void* out_bf16, int T, int inner, int groups, hipStream_t stream) {
   LGA_CHECK_ARG(y && z && w && out && T > 0 && inner > 0, "lgs_gated_group_norm: bad arguments");
-  LGA_CHECK_ARG(groups > 0 && groups <= 65535 && inner % groups == 0, "lgs_gated_group_norm: inner must divide into the groups");
+  LGA_CHECK_ARG(groups > 0 && groups <= 65535 && inner % groups == 0,
+                "lgs_gated_group_norm: inner must divide into the groups");
   lgs::gated_group_norm_kernel<<<dim3(T, groups), 256, 0, stream>>>(y, z, ldz, w, eps, out, (uint16_t*)out_bf16,
                                                                    inner / groups, inner);
   LGA_LAUNCH_RETURN();

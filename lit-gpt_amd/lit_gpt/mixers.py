@@ -229,8 +229,8 @@ class DiffAttention(InputReader):
 
 
 class SelectiveScan(InputReader):
-    """Selective state-space mixer in the Mamba-2 form. One input projection whose rows are ordered [z | x | B | C | dt] (inner =
-    heads * vdim gate and value columns, groups * state columns each for B and C, one step size per head); x, B and C
+    """Selective state-space mixer in the Mamba-2 form. One input projection whose rows are ordered
+    [z | x | B | C | dt] (inner = heads * vdim gate and value columns, groups * state columns each for B and C, one step size per head); x, B and C
     pass a short causal per-channel convolution and silu; dt = softplus(dt + bias); per head (heads share B and C in
     groups) S_t = exp(-exp(A_log) dt_t) S_{t-1} + dt_t B_t x_t^T, y_t = S_t^T C_t + D x_t; y is gated with silu(z),
     divided by its root mean square in ``norm_groups`` equal parts, weighted and projected. The state (S and the

@@ -455,8 +455,8 @@ def diffattn(proj: torch.Tensor, q_off: int, cache_k: torch.Tensor, cache_v: tor
 def conv_silu(proj: torch.Tensor, off: int, weight: torch.Tensor, bias: torch.Tensor, state: torch.Tensor,
               seq_start: torch.Tensor, seq_slot: torch.Tensor, seq_pos0: torch.Tensor, max_len: int) -> torch.Tensor:
     """silu(causal per-channel convolution + bias) of the C columns of ``proj`` at ``off`` over a packed batch;
-    weight (C, taps): column taps - 1 weights the token itself, column 0 the oldest input. state (slots, taps - 1, C) fp32 carries every sequence's last
-    inputs from step to step. Returns (T, C) fp32."""
+    weight (C, taps): column taps - 1 weights the token itself, column 0 the oldest input. state (slots, taps - 1, C)
+    fp32 carries every sequence's last inputs from step to step. Returns (T, C) fp32."""
     T, ld = proj.shape
     C, taps = weight.shape
     B = seq_slot.numel()

@@ -44,7 +44,7 @@ def softplus(z: torch.Tensor) -> torch.Tensor:
 
 
 def rope_interleaved(x: torch.Tensor, pos: int, dims: int, base: float) -> torch.Tensor:
-    """Rotate the first ``dims`` entries of a vector, entry 2i paired with entry 2i + 1; entries from ``dims`` on are copied."""
+    """Rotate the first ``dims`` entries of a vector, entry 2i paired with entry 2i + 1; the others are copied."""
     if dims == 0:
         return x.clone()
     i = torch.arange(dims // 2, dtype=x.dtype)
@@ -109,7 +109,8 @@ def diff_attention(h: torch.Tensor, w: Dict[str, torch.Tensor], m: dict, eps: fl
 
 
 def causal_conv(u: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
-    """Per-channel causal convolution: u (T, C), weight (C, taps): column taps - 1 weights the token itself, column 0 the oldest input."""
+    """Per-channel causal convolution of u (T, C) with weight (C, taps): column taps - 1 weights the token itself,
+    column 0 the oldest input."""
     T, C = u.shape
     taps = weight.shape[1]
     out = torch.zeros_like(u)
